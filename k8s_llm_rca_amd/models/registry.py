@@ -5,8 +5,9 @@ checkpoint folder's config.json.
 * ``opt``                 -- :class:`~.opt.OPTModel` (the CPU plumbing backend)
 * ``zasapel``             -- :class:`~.zasapel.ZasapelModel` (config.json with ``"architecture": "Zasapel"``)
 * ``ligipel``             -- :class:`~.ligipel.LigipelModel` (config.json with ``"architecture": "Ligipel"``)
+* ``lizesun``             -- :class:`~.lizesun.LizesunModel` (config.json with ``"architecture": "Lizesun"``)
 
-The last two describe their layers one by one in config.json (``OWN_CONFIG``): their
+The last three describe their layers one by one in config.json (``OWN_CONFIG``): their
 configuration objects are built from it, not from a preset with overrides.
 """
 from __future__ import annotations
@@ -19,7 +20,8 @@ from . import config as C
 
 
 # architectures whose config.json lists the layers (``"architecture": <name>``): module, model class
-OWN_CONFIG = {"zasapel": ("zasapel", "ZasapelModel"), "ligipel": ("ligipel", "LigipelModel")}
+OWN_CONFIG = {"zasapel": ("zasapel", "ZasapelModel"), "ligipel": ("ligipel", "LigipelModel"),
+              "lizesun": ("lizesun", "LizesunModel")}
 
 
 def _module(arch: str):

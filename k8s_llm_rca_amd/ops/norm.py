@@ -219,3 +219,58 @@ def softcap_(logits: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
     if cap > 0:
         logits.copy_(cap * torch.tanh(logits / cap))
     return logits
+
+
+# ------------------------------------------------------------------ Dynamic Tanh norm around an fp32 residual
+# (csrc/kernels/dyt_ops.hip).  ``dyt(x) = tanh(alpha x) * w + b`` per element: no mean, no variance, so
+# nothing couples a row's entries and the residual add, the norm and the cast are one elementwise pass.
+def embed_scale_dyt(ids: torch.Tensor, embed: torch.Tensor, scale: float, x_out: torch.Tensor, alpha: float,
+                    w: Optional[torch.Tensor], b: Optional[torch.Tensor], out_dtype) -> Optional[torch.Tensor]:
+    """``x_out = embed[ids] * scale`` (fp32); with ``w, b`` also returns ``dyt(x_out)`` as activations."""
+    T, W = ids.shape[0], embed.shape[1]
+    h = torch.empty(T, W, dtype=out_dtype, device=embed.device) if w is not None else None
+    if use_hip(embed):
+        assert x_out.dtype == torch.float32 and x_out.is_contiguous() and x_out.shape == (T, W)
+        assert embed.is_contiguous() and ids.dtype == torch.int32
+        check(lib().k8s_embed_scale_dyt(ptr(ids), ptr(embed), _odt(embed.dtype), float(scale), ptr(x_out),
+                                        float(alpha), ptr(w), ptr(b), ptr(h), _odt(out_dtype) if h is not None else 1,
+                                        T, W, stream_ptr(embed)), "embed_scale_dyt")
+        return h
+    x_out.copy_(embed[ids.long()].float() * scale)
+    if h is not None:
+        h.copy_((torch.tanh(alpha * x_out) * w + b).to(out_dtype))
+    return h
+
+
+def add_dyt(x: torch.Tensor, y: Optional[torch.Tensor], sy: float = 1.0, y2: Optional[torch.Tensor] = None,
+            sy2: float = 1.0, alpha: float = 1.0, w: Optional[torch.Tensor] = None, b: Optional[torch.Tensor] = None,
+            out_dtype=None) -> Optional[torch.Tensor]:
+    """In place on the fp32 residual: ``x += sy * y (+ sy2 * y2)`` (``y`` None: nothing is added); with
+    ``w, b`` also returns ``tanh(alpha x) * w + b`` of the new rows as activations (the next sublayer's
+    input norm, same pass)."""
+    T, W = x.shape
+    h = torch.empty(T, W, dtype=out_dtype, device=x.device) if w is not None else None
+    if use_hip(x):
+        for t in (x, y, y2):
+            assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.shape == (T, W))
+        assert y is not None or y2 is None
+        if y is None and h is None:
+            return None
+        check(lib().k8s_add_dyt(ptr(x), ptr(y), float(sy), ptr(y2), float(sy2), float(alpha), ptr(w), ptr(b), ptr(h),
+                                _odt(out_dtype) if h is not None else 1, T, W, stream_ptr(x)), "add_dyt")
+        return h
+    if y is not None:
+        x.add_(sy * y if y2 is None else sy * y + sy2 * y2)
+    if h is not None:
+        h.copy_((torch.tanh(alpha * x) * w + b).to(out_dtype))
+    return h
+
+
+def relu_sq(u: torch.Tensor) -> torch.Tensor:
+    """``max(u, 0)^2`` per element, in fp32, as ``u``'s type."""
+    if use_hip(u):
+        assert u.is_contiguous()
+        out = torch.empty_like(u)
+        check(lib().k8s_relu_sq(ptr(u), ptr(out), u.numel(), _odt(u.dtype), stream_ptr(u)), "relu_sq")
+        return out
+    return torch.relu(u.float()).pow(2).to(u.dtype)

@@ -1,7 +1,10 @@
 """Ops of layers that carry per-sequence state besides the paged cache:
 sinusoidal positions, the short causal convolution in front of a sublayer, the
-minGRU recurrence, the post-sublayer norm of an fp32 residual, and attention
-over a paged latent cache (``csrc/kernels/seq_ops.hip``, ``latent_attn.hip``).
+minGRU recurrence, the post-sublayer norm of an fp32 residual, attention over a
+paged latent cache (``csrc/kernels/seq_ops.hip``, ``latent_attn.hip``), window
+attention and recurrent mixers (``mixer_ops.hip``, ``window_attn.hip``), masked
+softmax attention behind a q / k preparation pass and matrix-state recurrences
+(``masked_attn.hip``, ``matrix_mem.hip``).
 
 A step's rows come in SEGMENTS (:class:`SegMeta`): consecutive rows of one
 sequence -- a decode token or a portion of a prompt.  Device tensors run the HIP
@@ -586,4 +589,265 @@ def window_attention(qkv: torch.Tensor, H: int, G: int, D: int, V: int, kc: torc
         p = ex / (torch.exp(-m) + ex.sum(-1, keepdim=True))
         pm = torch.einsum("hg,tgj->thj", talk, p)
         out[a:e] = torch.einsum("thj,jhv->thv", pm, v).reshape(n, H * V).to(qkv.dtype)
+    return out
+
+
+# ------------------------------------------------------------------ masked softmax attention with a prepared q / k,
+# and matrix-state recurrences (csrc/kernels/masked_attn.hip, matrix_mem.hip)
+def attn_prep(qkv: torch.Tensor, bias: Optional[torch.Tensor], H: int, G: int, D: int, V: int,
+              positions: torch.Tensor, slots: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, out_dtype,
+              norm: bool = False, q_w: Optional[torch.Tensor] = None, k_w: Optional[torch.Tensor] = None,
+              eps: float = 0.0, rot_dims: int = 0, rot_base: float = 10000.0, lam: float = 0.0,
+              v_other: Optional[torch.Tensor] = None, v_keep: Optional[torch.Tensor] = None,
+              vt: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Between the joint projection and attention, one pass over the fp32 rows of ``qkv`` [T, H D + G D + G V]
+    = (q | k | v):  add ``bias`` (fp32, same width, optional);  rotate q and k on their first ``rot_dims``
+    entries per head (entry i paired with i + rot_dims / 2, angle ``pos * rot_base^(-2 i / rot_dims)``);  with
+    ``norm`` divide every q and k head by its root mean square (``eps`` inside the root) and multiply by
+    ``q_w`` / ``k_w`` [D] where given;  ``v_keep`` [T, G V] fp32 receives the values as projected;  with
+    ``v_other`` the values become ``(1 - lam) v + lam v_other``.  k and v go to the pages ``kc`` [pages, BS, G D] /
+    ``vc`` [pages, BS, G V] at ``slots`` (and v to the transposed twin ``vt`` when given); q is returned
+    [T, H D] as activations."""
+    T = qkv.shape[0]
+    NQ, NK, NV = H * D, G * D, G * V
+    q_out = torch.empty(T, NQ, dtype=out_dtype, device=qkv.device)
+    BS = kc.shape[1]
+    if use_hip(qkv):
+        assert qkv.dtype == torch.float32 and qkv.stride(1) == 1 and qkv.shape[1] == NQ + NK + NV
+        assert kc.is_contiguous() and vc.is_contiguous() and kc.dtype == vc.dtype == out_dtype
+        assert kc.shape[-1] == NK and vc.shape[-1] == NV and rot_dims % 2 == 0 and 0 <= rot_dims <= D
+        for t in (bias, q_w, k_w):
+            assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+        for t in (v_other, v_keep):
+            assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.shape == (T, NV))
+        assert vt is None or (vt.is_contiguous() and vt.dtype == out_dtype and vt.shape[1:] == (NV, BS))
+        check(lib().k8s_attn_prep(ptr(qkv), qkv.stride(0), ptr(bias), H, G, D, V, ptr(positions), ptr(slots),
+                                  ptr(kc), ptr(vc), ptr(vt), BS, ptr(q_out), _dt(out_dtype), int(norm), ptr(q_w),
+                                  ptr(k_w), float(eps), int(rot_dims), float(rot_base), float(lam), ptr(v_other),
+                                  ptr(v_keep), T, stream_ptr(qkv)), "attn_prep")
+        return q_out
+    x = qkv + bias if bias is not None else qkv
+    q, k, v = x[:, :NQ].reshape(T, H, D), x[:, NQ:NQ + NK].reshape(T, G, D), x[:, NQ + NK:]
+    if rot_dims:
+        half = rot_dims // 2
+        f = torch.exp(-(2.0 * torch.arange(half, dtype=torch.float64) / rot_dims) * math.log(rot_base))
+        ang = positions.double()[:, None] * f[None]
+        co, si = ang.cos().float()[:, None, :], ang.sin().float()[:, None, :]
+
+        def rot(z):
+            a, b = z[..., :half], z[..., half:rot_dims]
+            return torch.cat([a * co - b * si, b * co + a * si, z[..., rot_dims:]], -1)
+
+        q, k = rot(q), rot(k)
+    if norm:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
+        if q_w is not None:
+            q = q * q_w
+        if k_w is not None:
+            k = k * k_w
+    if v_keep is not None:
+        v_keep.copy_(v)
+    if v_other is not None:
+        v = (1.0 - lam) * v + lam * v_other
+    ok = slots >= 0
+    sl = slots[ok].long()
+    kc.view(-1, NK)[sl] = k.reshape(T, NK)[ok].to(kc.dtype)
+    vc.view(-1, NV)[sl] = v[ok].to(vc.dtype)
+    if vt is not None:
+        vt[sl // BS, :, sl % BS] = v[ok].to(vt.dtype)
+    q_out.copy_(q.reshape(T, NQ).to(out_dtype))
+    return q_out
+
+
+def masked_attention(q: torch.Tensor, H: int, G: int, D: int, V: int, kc: torch.Tensor, vc: torch.Tensor,
+                     seg: SegMeta, scale: float, softcap: float = 0.0, chunk: int = 0, window: int = 0,
+                     keep_first: int = 0, sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                     vt: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Softmax attention of the rows' queries ``q`` [T, H D] over the paged keys and values (which already
+    hold this step's rows), query head h reading key / value head ``h // (H // G)``.  Position i sees j <= i
+    with, for ``chunk`` > 0, ``i // chunk == j // chunk`` and, for ``window`` > 0, ``i - j < window or j < keep_first``
+    (positions count from the sequence's start).  ``s = scale q.k``, then ``softcap * tanh(s / softcap)`` for
+    ``softcap`` > 0.  ``sink`` [H] fp32 adds ``exp(sink_h)`` to head h's denominator (no key, no value).  ``gate``
+    [T, >= H] fp32 (row stride free): head h's output is multiplied by ``sigmoid(gate[t, h])``.
+    Returns [T, H V].  With the transposed value pages ``vt`` (bf16, sizes of :func:`masked_mfma_ok`) the
+    matrix-core kernel runs."""
+    T = q.shape[0]
+    BS = kc.shape[1]
+    out = torch.empty(T, H * V, dtype=q.dtype, device=q.device)
+    if use_hip(q):
+        assert q.is_contiguous() and q.shape[1] == H * D and kc.is_contiguous() and vc.is_contiguous()
+        assert kc.dtype == vc.dtype == q.dtype and kc.shape[-1] == G * D and vc.shape[-1] == G * V and H % G == 0
+        assert seg.block_tables.is_contiguous() and chunk >= 0 and window >= 0 and keep_first >= 0
+        assert sink is None or (sink.dtype == torch.float32 and sink.shape[0] == H)
+        assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.shape[1] >= H)
+        gs = gate.stride(0) if gate is not None else 0
+        if vt is not None and masked_mfma_ok(H, G, D, V, q.dtype, q.device):
+            assert vt.is_contiguous() and vt.shape[1:] == (G * V, BS) and BS % 32 == 0
+            items = seg.tile_items(WINDOW_TILE)
+            check(lib().k8s_masked_attn_mfma(ptr(q), ptr(kc), ptr(vt), ptr(seg.block_tables),
+                                             seg.block_tables.shape[1], ptr(items), items.shape[0], ptr(sink),
+                                             ptr(gate), gs, ptr(out), H, G, D, V, BS, int(chunk), int(window),
+                                             int(keep_first), float(scale), float(softcap), stream_ptr(q)),
+                  "masked_attn_mfma")
+            return out
+        check(lib().k8s_masked_attn_rows(ptr(q), ptr(kc), ptr(vc), ptr(seg.block_tables), seg.block_tables.shape[1],
+                                         ptr(seg.row_seg), ptr(seg.seg_row0), ptr(seg.seg_pos0), ptr(sink), ptr(gate),
+                                         gs, ptr(out), T, H, G, D, V, BS, int(chunk), int(window), int(keep_first),
+                                         float(scale), float(softcap), _dt(q.dtype), stream_ptr(q)),
+              "masked_attn_rows")
+        return out
+    kf, vf = kc.view(-1, G, D), vc.view(-1, G, V)
+    rep = H // G
+    for s in range(seg.n_seg):
+        a, e, p0 = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s]
+        n, n_ctx = e - a, p0 + e - a
+        kp = torch.arange(n_ctx)
+        rows = seg.block_tables[s].long()[kp // BS] * BS + kp % BS
+        k = kf[rows].float().repeat_interleave(rep, 1)             # [ctx, H, D]
+        v = vf[rows].float().repeat_interleave(rep, 1)             # [ctx, H, V]
+        qi = (p0 + torch.arange(n))[:, None]
+        vis = kp[None, :] <= qi
+        if chunk > 0:
+            vis &= (qi // chunk) == (kp[None, :] // chunk)
+        if window > 0:
+            vis &= ((qi - kp[None, :]) < window) | (kp[None, :] < keep_first)
+        sc = torch.einsum("thd,jhd->thj", q[a:e].float().view(n, H, D), k) * scale
+        if softcap > 0:
+            sc = softcap * torch.tanh(sc / softcap)
+        sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
+        m = sc.amax(-1, keepdim=True)
+        if sink is not None:
+            m = torch.maximum(m, sink[None, :, None])
+        ex = torch.exp(sc - m)
+        den = ex.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sink[None, :, None] - m)
+        o = torch.einsum("thj,jhv->thv", ex / den, v)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[a:e, :H])[:, :, None]
+        out[a:e] = o.reshape(n, H * V).to(q.dtype)
+    return out
+
+
+def masked_mfma_ok(H: int, G: int, D: int, V: int, dtype, device) -> bool:
+    """Whether the matrix-core form of :func:`masked_attention` takes these sizes (bf16 on the device only)."""
+    if dtype != torch.bfloat16 or torch.device(device).type != "cuda":
+        return False
+    fn = getattr(lib(), "k8s_masked_attn_mfma_ok", None)
+    return bool(fn(int(H), int(G), int(D), int(V))) if fn is not None else False
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, H: int, V: int, eps: float,
+                   out_dtype) -> torch.Tensor:
+    """``o / rms(o over each head's V) * w * sigmoid(gate)`` of fp32 rows ``o`` [T, H V]; ``w`` [V] (shared by the
+    heads) or [H V]; ``gate`` [T, H V] fp32 (row stride free)."""
+    T = o.shape[0]
+    out = torch.empty(T, H * V, dtype=out_dtype, device=o.device)
+    if use_hip(o):
+        assert o.dtype == gate.dtype == w.dtype == torch.float32 and o.is_contiguous() and gate.stride(1) == 1
+        assert w.numel() in (V, H * V)
+        check(lib().k8s_head_norm_gate(ptr(o), ptr(gate), gate.stride(0), ptr(w), V if w.numel() == H * V else 0,
+                                       ptr(out), T, H, V, float(eps), _dt(out_dtype), stream_ptr(o)), "head_norm_gate")
+        return out
+    oh = o.view(T, H, V)
+    oh = oh * torch.rsqrt(oh.pow(2).mean(-1, keepdim=True) + eps)
+    wv = w.view(H, V) if w.numel() == H * V else w.view(1, V)
+    out.copy_((oh * wv * torch.sigmoid(gate[:, :H * V]).view(T, H, V)).reshape(T, H * V).to(out_dtype))
+    return out
+
+
+UNIT_EPS = 1e-6     # q and k of the delta rule: x / sqrt(sum(x^2) + UNIT_EPS)
+
+
+def gated_delta(qkv: torch.Tensor, H: int, G: int, D: int, V: int, a: torch.Tensor, rate: torch.Tensor,
+                dt_bias: torch.Tensor, beta: torch.Tensor, state: torch.Tensor, seg: SegMeta) -> torch.Tensor:
+    """Gated delta rule per head, fp32.  Rows of ``qkv`` [T, 2 G D + H V] = (q | k | v) activations; head h
+    reads q / k head ``h // (H // G)``; q and k become unit vectors (``UNIT_EPS``), q times ``D^(-1/2)``.
+    Decay per head and key channel ``g = exp(-rate_h softplus(a + dt_bias))`` from ``a`` [T, H D] fp32;
+    ``beta`` [T, >= H] fp32 before its sigmoid (row stride free).  Per token
+    ``S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q`` with ``S`` [D, V].
+    ``state`` [slots, H, D, V] fp32 is read (past position 0) and advanced.  Returns o [T, H V] fp32."""
+    T = qkv.shape[0]
+    out = torch.empty(T, H * V, dtype=torch.float32, device=qkv.device)
+    if use_hip(qkv):
+        assert qkv.is_contiguous() and qkv.shape[1] == 2 * G * D + H * V and H % G == 0
+        assert a.dtype == torch.float32 and a.is_contiguous() and a.shape == (T, H * D)
+        assert beta.dtype == torch.float32 and beta.stride(1) == 1 and beta.shape[1] >= H
+        assert rate.dtype == dt_bias.dtype == torch.float32 and rate.numel() == H and dt_bias.numel() == H * D
+        assert state.is_contiguous() and state.shape[1:] == (H, D, V)
+        check(lib().k8s_gated_delta(ptr(qkv), _dt(qkv.dtype), ptr(a), ptr(rate), ptr(dt_bias), ptr(beta),
+                                    beta.stride(0), ptr(state), ptr(seg.seg_row0), ptr(seg.seg_pos0),
+                                    ptr(seg.seg_slot), ptr(out), seg.n_seg, T, H, G, D, V, float(UNIT_EPS),
+                                    stream_ptr(qkv)), "gated_delta")
+        return out
+    x = qkv.float()
+    q = x[:, :G * D].view(T, G, D)
+    k = x[:, G * D:2 * G * D].view(T, G, D)
+    v = x[:, 2 * G * D:].view(T, H, V)
+    q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + UNIT_EPS) * D ** -0.5
+    k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + UNIT_EPS)
+    rep = H // G
+    q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)      # [T, H, D]
+    g = torch.exp(-rate.view(1, H, 1) * torch.nn.functional.softplus(a + dt_bias.view(1, -1)).view(T, H, D))
+    bt = torch.sigmoid(beta[:, :H])
+    for s in range(seg.n_seg):
+        r0, r1, p0, sl = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s], seg.slot_host[s]
+        S = state[sl].clone() if p0 > 0 else torch.zeros(H, D, V)
+        for r in range(r0, r1):
+            S = g[r][:, :, None] * S
+            u = bt[r][:, None] * (v[r] - torch.einsum("hdv,hd->hv", S, k[r]))
+            S = S + k[r][:, :, None] * u[:, None, :]
+            out[r] = torch.einsum("hdv,hd->hv", S, q[r]).reshape(-1)
+        state[sl] = S
+    return out
+
+
+DEN_EPS = 1e-6      # matrix memory: o = S^T q / (max(|n.q|, exp(-m)) + DEN_EPS)
+
+
+def matrix_memory(x: torch.Tensor, H: int, D: int, V: int, gate_bias: torch.Tensor, cap: float,
+                  state: torch.Tensor, nstate: torch.Tensor, mstate: torch.Tensor, seg: SegMeta) -> torch.Tensor:
+    """Matrix memory with exponential gates per head, fp32.  Rows of ``x`` [T, 2 H D + 2 H V + 2 H] fp32 =
+    (q | k | v | . | i | f): q is scaled by ``D^(-1/2)``; the log gates are ``i = cap tanh((i + b_i) / cap)`` and
+    ``f = logsigmoid(cap tanh((f + b_f) / cap))`` with ``gate_bias`` [2 H] = (b_i | b_f).  With the running maximum
+    ``m`` (0 at the start of a sequence):  ``m' = max(f + m, i)``;  ``S <- e^(f + m - m') S + e^(i - m') k v^T``;  n likewise
+    with k alone;  ``o = S^T q / (max(|n.q|, e^(-m')) + DEN_EPS)``.  ``state`` [slots, H, D, V], ``nstate`` [slots, H, D],
+    ``mstate`` [slots, H] fp32 are read (past position 0) and advanced.  Returns o [T, H V] fp32."""
+    T = x.shape[0]
+    out = torch.empty(T, H * V, dtype=torch.float32, device=x.device)
+    if use_hip(x):
+        assert x.dtype == torch.float32 and x.stride(1) == 1 and x.shape[1] == 2 * H * (D + V) + 2 * H
+        assert gate_bias.dtype == torch.float32 and gate_bias.numel() == 2 * H
+        assert state.is_contiguous() and state.shape[1:] == (H, D, V) and nstate.is_contiguous()
+        assert nstate.shape[1:] == (H, D) and mstate.is_contiguous() and mstate.shape[1:] == (H,)
+        ab = scratch(T * H * 3, torch.float32, x.device)
+        check(lib().k8s_matrix_memory(ptr(x), x.stride(0), ptr(gate_bias), float(cap), ptr(state), ptr(nstate),
+                                      ptr(mstate), ptr(seg.seg_row0), ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(ab),
+                                      ptr(out), seg.n_seg, T, H, D, V, float(DEN_EPS), stream_ptr(x)),
+              "matrix_memory")
+        return out
+    HD, HV = H * D, H * V
+    q = x[:, :HD].view(T, H, D) * D ** -0.5
+    k = x[:, HD:2 * HD].view(T, H, D)
+    v = x[:, 2 * HD:2 * HD + HV].view(T, H, V)
+    gi = x[:, 2 * HD + 2 * HV:2 * HD + 2 * HV + H] + gate_bias[:H]
+    gf = x[:, 2 * HD + 2 * HV + H:] + gate_bias[H:]
+    gi = cap * torch.tanh(gi / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh(gf / cap))
+    for s in range(seg.n_seg):
+        r0, r1, p0, sl = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s], seg.slot_host[s]
+        if p0 > 0:
+            S, n, m = state[sl].clone(), nstate[sl].clone(), mstate[sl].clone()
+        else:
+            S, n, m = torch.zeros(H, D, V), torch.zeros(H, D), torch.zeros(H)
+        for r in range(r0, r1):
+            mn = torch.maximum(gf[r] + m, gi[r])
+            fa, ia = torch.exp(gf[r] + m - mn), torch.exp(gi[r] - mn)
+            S = fa[:, None, None] * S + ia[:, None, None] * k[r][:, :, None] * v[r][:, None, :]
+            n = fa[:, None] * n + ia[:, None] * k[r]
+            m = mn
+            den = torch.maximum((n * q[r]).sum(-1).abs(), torch.exp(-m)) + DEN_EPS
+            out[r] = (torch.einsum("hdv,hd->hv", S, q[r]) / den[:, None]).reshape(-1)
+        state[sl], nstate[sl], mstate[sl] = S, n, m
     return out
