@@ -109,6 +109,16 @@ _SIGS = {
     "k8s_window_attn_mfma_ok": [I, I, I, I],
     "k8s_window_attn_mfma": [P, I, P, P, P, I, P, I, P, P, P, P, I, I, I, I, I, I, F, P, I, I, P, P],
     "k8s_window_attn_rows": [P, I, P, P, P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
+    "k8s_add_dyt": [P, P, F, P, F, F, P, P, P, I, I, I, P],
+    "k8s_embed_scale_dyt": [P, P, I, F, P, F, P, P, P, I, I, I, P],
+    "k8s_relu_sq": [P, P, ctypes.c_long, I, P],
+    "k8s_attn_prep": [P, I, P, I, I, I, I, P, P, P, P, P, I, P, I, I, P, P, F, I, F, F, P, P, I, P],
+    "k8s_masked_attn_rows": [P, P, P, P, I, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, I, F, F, I, P],
+    "k8s_masked_attn_mfma_ok": [I, I, I, I],
+    "k8s_masked_attn_mfma": [P, P, P, P, I, P, I, P, P, I, P, I, I, I, I, I, I, I, I, F, F, P],
+    "k8s_gated_delta": [P, I, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, P],
+    "k8s_matrix_memory": [P, I, P, F, P, P, P, P, P, P, P, P, I, I, I, I, I, F, P],
+    "k8s_head_norm_gate": [P, P, I, P, I, P, I, I, I, F, I, P],
     "k8s_walks": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
 }
 # entry points whose C return type is not int
