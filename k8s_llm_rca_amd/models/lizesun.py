@@ -236,8 +236,8 @@ class LizesunModel:
                 self.cache_of.append(None)
             if L.kind == "attention" and a.v_mix:
                 if self.vmix_first is None:
-                    self.vmix_first, vmix_width = i, a.kv_heads * a.vdim
-                elif a.kv_heads * a.vdim != vmix_width:
+                    self.vmix_first, vmix_width = i, (a.kv_heads, a.vdim)
+                elif (a.kv_heads, a.vdim) != vmix_width:
                     raise ValueError(f"layer {i}: layers that mix values must have values of one size")
             if L.kind == "parallel":
                 if L.left.rot_dims % 2 or L.left.rot_dims > L.left.dim:

@@ -72,8 +72,8 @@ def chunked_attention(h, t, p, m, eps, v_first):
         else:
             lam = t[p + "vmix"]
             v = (1.0 - lam) * v + lam * v_first
-    c = int(m["mask"]["size"])
-    o = masked_softmax_attention(q, k, v, float(m["scale"]), lambda i, j: i // c == j // c,
+    c = int((m.get("mask") or {}).get("size", 0))        # no mask: plain causal
+    o = masked_softmax_attention(q, k, v, float(m["scale"]), lambda i, j: not c or i // c == j // c,
                                  softcap=float(m.get("softcap") or 0.0))
     o = o * torch.sigmoid(h @ t[p + "g"].T)[:, :, None]
     return o.reshape(n, H * V) @ t[p + "o"].T, mine
@@ -84,12 +84,15 @@ def window_sink_attention(h, t, p, m, eps):
     n = h.shape[0]
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     pos = torch.arange(n)
-    q = rotate_half((h @ t[p + "q"].T).view(n, H, D), pos, int(m["rot"]["dims"]), float(m["rot"]["base"]))
-    k = rotate_half((h @ t[p + "k"].T).view(n, G, D), pos, int(m["rot"]["dims"]), float(m["rot"]["base"]))
+    rot = m.get("rot") or {"dims": 0, "base": 1.0}       # no rot: no rotation
+    q = rotate_half((h @ t[p + "q"].T).view(n, H, D), pos, int(rot["dims"]), float(rot["base"]))
+    k = rotate_half((h @ t[p + "k"].T).view(n, G, D), pos, int(rot["dims"]), float(rot["base"]))
     v = (h @ t[p + "v"].T).view(n, G, V)
     q, k = unit_rms(q, eps), unit_rms(k, eps)
-    w, kf = int(m["mask"]["size"]), int(m["mask"].get("keep_first", 0))
-    o = masked_softmax_attention(q, k, v, float(m["scale"]), lambda i, j: i - j < w or j < kf, sink=t[p + "sink"])
+    mask = m.get("mask") or {}
+    w, kf = int(mask.get("size", 0)), int(mask.get("keep_first", 0))
+    o = masked_softmax_attention(q, k, v, float(m["scale"]), lambda i, j: not w or i - j < w or j < kf,
+                                 sink=t[p + "sink"])
     return o.reshape(n, H * V) @ t[p + "o"].T
 
 
