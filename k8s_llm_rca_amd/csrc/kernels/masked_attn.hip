@@ -231,6 +231,185 @@ __global__ void __launch_bounds__(256) masked_attn_rows_kernel(const TA* __restr
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Matrix-core form (bf16, v_mfma_f32_16x16x32_bf16), one pass with an online softmax.  A work item is a
+// tile of up to 16 consecutive tokens of one segment; wave w of workgroup (item, y) owns the heads
+// (8 y + w) HW .. + HW - 1 and shares nothing with the other waves (no LDS, no barrier).  Keys go in
+// blocks of 32 that never cross a page (BS % 32 == 0): first the blocks that hold kept first tokens, then
+// the blocks from the first token's window / chunk start to the tile's last position; the exact mask is
+// applied per (query, key).  Swapped QK^T as in the other attention kernels: a lane owns ONE query
+// (lane & 15) and per block the scores of keys 8 q .. 8 q + 7 of its quarter q = lane >> 4, which is the
+// layout of the PV product's first operand, so the weights go from accumulator to operand in place.
+// The output accumulator's rows are the queries 4 q + i: their rescaling factors come from the lanes
+// that own those queries by a cross-lane read.
+struct MaskArgs {
+  const uint16_t* q;      // [T][H * D]
+  const uint16_t* kc;     // [pages][BS][G * D]
+  const uint16_t* vt;     // [pages][G * V][BS]
+  const int* bt;
+  int maxb;
+  const int* items;       // [n][4]: segment, first row, tokens (<= 16), position of the first token
+  const float* sink;      // [H] or null
+  const float* gate;      // [T] rows of stride gs, column h, or null
+  int gs;
+  uint16_t* out;          // [T][H * V]
+  int H, G, BS, chunk, window, keep_first;
+  float scale, softcap;
+};
+
+__device__ __forceinline__ bf16x8 mld16(const uint16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+
+template <int NDC, int NV, int HW>
+__global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
+  constexpr int D = NDC * 32, V = NV * 16;
+  constexpr float kLog2e = 1.4426950408889634f;
+  const int lane = threadIdx.x & 63, r = lane & 15, hq = lane >> 4;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int item = blockIdx.x;
+  const int sg = a.items[item * 4], row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2],
+            pos0 = a.items[item * 4 + 3];
+  const int H = a.H, hpg = H / a.G, NK = a.G * D, NVt = a.G * V;
+  const int h0 = (blockIdx.y * 8 + wv) * HW, nh = min(HW, H - h0);
+  if (nh <= 0) return;                                     // the whole wave; nothing below synchronises waves
+  const int posq = pos0 + r, pos_last = pos0 + ntok - 1;
+  const bool qvalid = r < ntok;
+  // this query's own bounds
+  const int cq_lo = a.chunk > 0 ? (posq / a.chunk) * a.chunk : 0;
+  const int wq_lo = a.window > 0 ? posq - a.window + 1 : 0;
+  const int keep = a.window > 0 ? a.keep_first : 0;
+  // the tile's key blocks: [a_beg, a_end) (kept first tokens) and [lo_al, pos_last]
+  const KeyRuns k0 = key_runs(pos0, a.chunk, a.window, a.keep_first);
+  const int lo_al = k0.lo & ~31, a_beg = k0.a0 & ~31;
+  const int a_end = a.window > 0 ? min(lo_al, (a.keep_first + 31) & ~31) : a_beg;
+  const int nblkA = max(0, (a_end - a_beg) >> 5), nblk = nblkA + ((pos_last - lo_al) >> 5) + 1;
+  const int* pages = a.bt + (size_t)sg * a.maxb;
+  bf16x8 qf[HW][NDC];
+  float m2[HW], l[HW];
+  f32x4 o[HW][NV];
+#pragma unroll
+  for (int hh = 0; hh < HW; ++hh) {
+    const bool on = hh < nh && qvalid;
+    const uint16_t* qp = a.q + (size_t)(row0 + (on ? r : 0)) * H * D + (size_t)(on ? h0 + hh : 0) * D;
+#pragma unroll
+    for (int cc = 0; cc < NDC; ++cc) {
+      qf[hh][cc] = mld16(qp + 32 * cc + 8 * hq);
+      if (!on)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[hh][cc][j] = (__bf16)0.f;
+    }
+    m2[hh] = (a.sink && hh < nh) ? a.sink[h0 + hh] * kLog2e : -INFINITY;
+    l[hh] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float sc2 = a.scale * kLog2e, cap2 = a.softcap * kLog2e, icap = a.softcap > 0.f ? a.scale / a.softcap : 0.f;
+  for (int bi = 0; bi < nblk; ++bi) {
+    const int kb = bi < nblkA ? a_beg + 32 * bi : lo_al + 32 * (bi - nblkA);
+    const int page = pages[kb / a.BS], off = kb % a.BS;
+    const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK;
+    bf16x8 kf[2][NDC];
+    bf16x8 vf[NV];
+    int gprev = -1;
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      if (hh < nh) {
+        const int g = (h0 + hh) / hpg;
+        if (g != gprev) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const int key = 8 * (r >> 2) + 4 * t + (r & 3);
+#pragma unroll
+            for (int cc = 0; cc < NDC; ++cc) kf[t][cc] = mld16(kp + (size_t)key * NK + g * D + 32 * cc + 8 * hq);
+          }
+          const uint16_t* vp = a.vt + ((size_t)page * NVt + (size_t)g * V) * a.BS + off + 8 * hq;
+#pragma unroll
+          for (int dt = 0; dt < NV; ++dt) vf[dt] = mld16(vp + (size_t)(16 * dt + r) * a.BS);
+          gprev = g;
+        }
+        float p[8];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int cc = 0; cc < NDC; ++cc)
+            sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][cc], qf[hh][cc], sacc, 0, 0, 0);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = kb + 8 * hq + 4 * t + i;
+            const bool ok = qvalid && key <= posq && key >= cq_lo && (key >= wq_lo || key < keep);
+            float s2;
+            if (a.softcap > 0.f) {
+              // cap tanh(x), tanh(x) = 1 - 2 / (1 + e^(2x)), in log2 units
+              const float e = __builtin_amdgcn_exp2f(fminf(sacc[i] * icap * (2.f * kLog2e), 60.f));
+              s2 = cap2 * (1.f - 2.f / (1.f + e));
+            } else {
+              s2 = sacc[i] * sc2;
+            }
+            p[4 * t + i] = ok ? s2 : -INFINITY;
+          }
+        }
+        float cmax = p[0];
+#pragma unroll
+        for (int j = 1; j < 8; ++j) cmax = fmaxf(cmax, p[j]);
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+        const float mn = fmaxf(m2[hh], cmax);
+        const float ms = mn == -INFINITY ? 0.f : mn;       // a query that has seen no key yet
+        const float alpha = __builtin_amdgcn_exp2f(m2[hh] - ms);
+        float ps = 0.f;
+        bf16x8 pf;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float e = __builtin_amdgcn_exp2f(p[j] - ms);
+          ps += e;
+          pf[j] = (__bf16)e;
+        }
+        l[hh] = l[hh] * alpha + ps;
+        m2[hh] = mn;
+        float ai[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ai[i] = __shfl(alpha, 4 * hq + i, 64);
+#pragma unroll
+        for (int dt = 0; dt < NV; ++dt) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[hh][dt][i] *= ai[i];
+          o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[dt], o[hh][dt], 0, 0, 0);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int hh = 0; hh < HW; ++hh) {
+    if (hh < nh) {
+      float lt = l[hh];
+      lt += __shfl_xor(lt, 16, 64);
+      lt += __shfl_xor(lt, 32, 64);
+      if (a.sink) lt += __builtin_amdgcn_exp2f(a.sink[h0 + hh] * kLog2e - m2[hh]);
+      const float inv = 1.f / lt;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int qi = 4 * hq + i;
+        float f = __shfl(inv, qi, 64);
+        if (qi < ntok) {
+          if (a.gate) f *= 1.f / (1.f + __expf(-a.gate[(size_t)(row0 + qi) * a.gs + h0 + hh]));
+          uint16_t* op = a.out + (size_t)(row0 + qi) * H * V + (size_t)(h0 + hh) * V + r;
+#pragma unroll
+          for (int dt = 0; dt < NV; ++dt) op[16 * dt] = f2bf(o[hh][dt][i] * f);
+        }
+      }
+    }
+  }
+}
+
+template <int NDC, int NV>
+static int launch_mask_mfma(const MaskArgs& a, int n_items, hipStream_t s) {
+  constexpr int HW = 2;
+  const int waves_all = (a.H + HW - 1) / HW;               // two heads per wave, up to eight waves per workgroup
+  const int gy = (waves_all + 7) / 8, waves = gy > 1 ? 8 : waves_all;
+  hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW>), dim3(n_items, gy), dim3(64 * waves), 0, s, a);
+  return (int)hipGetLastError();
+}
+
 }  // namespace k8s
 
 using namespace k8s;
@@ -273,4 +452,41 @@ K8S_API int k8s_masked_attn_rows(const void* q, const void* kc, const void* vc, 
                        (const float*)vc, block_tables, maxb, row_seg, seg_row0, seg_pos0, sink, gate, gs, (float*)out, H,
                        G, D, V, BS, chunk, window, keep_first, scale, softcap);
   return (int)hipGetLastError();
+}
+
+// 1 when the matrix-core kernel takes these sizes (bf16 only)
+K8S_API int k8s_masked_attn_mfma_ok(int H, int G, int D, int V) {
+  return H >= 1 && G >= 1 && H % G == 0 && (D == 64 || D == 128) && (V == 64 || V == 128);
+}
+
+K8S_API int k8s_masked_attn_mfma(const void* q, const void* kc, const void* vt, const int* block_tables, int maxb,
+                                 const int* items, int n_items, const float* sink, const float* gate, int gs, void* out,
+                                 int H, int G, int D, int V, int BS, int chunk, int window, int keep_first, float scale,
+                                 float softcap, hipStream_t s) {
+  if (n_items <= 0) return 0;
+  if (!k8s_masked_attn_mfma_ok(H, G, D, V) || BS % 32 || chunk < 0 || window < 0 || keep_first < 0)
+    return (int)hipErrorInvalidValue;
+  MaskArgs a;
+  a.q = (const uint16_t*)q;
+  a.kc = (const uint16_t*)kc;
+  a.vt = (const uint16_t*)vt;
+  a.bt = block_tables;
+  a.maxb = maxb;
+  a.items = items;
+  a.sink = sink;
+  a.gate = gate;
+  a.gs = gs;
+  a.out = (uint16_t*)out;
+  a.H = H;
+  a.G = G;
+  a.BS = BS;
+  a.chunk = chunk;
+  a.window = window;
+  a.keep_first = keep_first;
+  a.scale = scale;
+  a.softcap = softcap;
+  if (D == 64 && V == 64) return launch_mask_mfma<2, 4>(a, n_items, s);
+  if (D == 64 && V == 128) return launch_mask_mfma<2, 8>(a, n_items, s);
+  if (D == 128 && V == 64) return launch_mask_mfma<4, 4>(a, n_items, s);
+  return launch_mask_mfma<4, 8>(a, n_items, s);
 }

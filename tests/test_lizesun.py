@@ -155,7 +155,7 @@ def engine(d, W, backend, num_blocks=24, block_size=32, slots=4, **kw):
     for t in eng.states.t.values():       # a fresh slot must not be read: make a read loud
         t.fill_(float("nan"))
     for c in eng.kv.kc + eng.kv.vc + [t for t in eng.kv.vt if t is not None]:
-        c.fill_(3e4)                      # stale pages hold finite garbage (a masked key is never read)
+        c.fill_(STALE)                    # stale pages hold finite garbage (a masked key's weight is 0)
     return eng
 
 
@@ -237,10 +237,13 @@ def test_dynamic_tanh_residual_pass_and_squared_relu(backend, W):
     close(N.relu_sq(u.to(dev).to(dt)), torch.relu(u) ** 2, dt)
 
 
+STALE = 2.0 ** 15     # what unwritten page entries hold in these tests (exact in bfloat16)
+
+
 def paged(dev, dt, n_pages, BS, G, D, V, order):
     """Empty key / value pages and a block table that walks them in ``order``."""
-    kc = torch.full((n_pages, BS, G * D), 3e4, device=dev, dtype=dt)
-    vc = torch.full((n_pages, BS, G * V), 3e4, device=dev, dtype=dt)
+    kc = torch.full((n_pages, BS, G * D), STALE, device=dev, dtype=dt)
+    vc = torch.full((n_pages, BS, G * V), STALE, device=dev, dtype=dt)
     return kc, vc, [list(order)]
 
 
@@ -272,7 +275,7 @@ def test_attention_preparation(backend, H, G, D, V, rot, norm, wts):
     v = xb[:, H * D + G * D:]
     order = [2, 0, 1]
     kc, vc, _ = paged(dev, dt, 3, BS, G, D, V, order)
-    vt = torch.full((3, G * V, BS), 3e4, device=dev, dtype=dt)
+    vt = torch.full((3, G * V, BS), STALE, device=dev, dtype=dt)
     sl = torch.tensor([order[i // BS] * BS + i % BS for i in range(T)], dtype=torch.int32, device=dev)
     f32 = lambda z: None if z is None else z.float().to(dev)  # noqa: E731
     keep = torch.empty(T, G * V, device=dev)
@@ -285,10 +288,10 @@ def test_attention_preparation(backend, H, G, D, V, rot, norm, wts):
     vm = (1 - lam) * v + lam * vo
     close(vc.view(-1, G * V)[sl.long()], vm, dt)
     close(vt[sl.long() // BS, :, sl.long() % BS], vm, dt)
-    assert float(kc[1].float().min()) == 3e4 and float(vc[0, 1:].float().min()) == 3e4   # nothing else was written
+    assert float(kc[1].float().min()) == STALE and float(vc[0, 1:].float().min()) == STALE   # nothing else was written
 
 
-def attention_case(dev, dt, H, G, D, V, n, BS, seed, sharp=None):
+def attention_case(dev, dt, H, G, D, V, n, BS, seed, sharp=None, with_twin=False):
     """Random q / k / v for one sequence, the keys and values in shuffled pages.  ``sharp`` = (i, j): key j is
     made to stand out for query i."""
     q, k, v = rnd(n, H, D, seed=seed), rnd(n, G, D, seed=seed + 1), rnd(n, G, V, seed=seed + 2)
@@ -303,6 +306,10 @@ def attention_case(dev, dt, H, G, D, V, n, BS, seed, sharp=None):
     sl = slots_of(order, BS, 0, n, dev).long()
     kc.view(-1, G * D)[sl] = k.reshape(n, -1).to(dev).to(dt)
     vc.view(-1, G * V)[sl] = v.reshape(n, -1).to(dev).to(dt)
+    if with_twin:                 # the values' transposed twin: the matrix-core kernel runs where it takes the sizes
+        vt = torch.full((n_pages + 2, G * V, BS), STALE, device=dev, dtype=dt)
+        vt[sl // BS, :, sl % BS] = v.reshape(n, -1).to(dev).to(dt)
+        return q, k, v, kc, vc, bt, vt
     return q, k, v, kc, vc, bt
 
 
@@ -339,6 +346,13 @@ def test_masked_attention_paged(backend, H, G, D, V, mask):
         close(in_portions(run, n, cuts), want.reshape(n, -1), dt)
 
 
+# query 100 and the key that stands out, just inside / outside every edge
+EDGES = {"chunk_in": (dict(chunk=26), 78), "chunk_out": (dict(chunk=26), 77),
+         "window_in": (dict(window=30, keep_first=4), 71), "window_out": (dict(window=30, keep_first=4), 70),
+         "first_in": (dict(window=30, keep_first=4), 3), "first_out": (dict(window=30, keep_first=4), 4),
+         "far": (dict(), 1)}
+
+
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("aim", ["chunk_in", "chunk_out", "window_in", "window_out", "first_in", "first_out", "far"])
 def test_one_key_stands_out_at_every_edge(backend, aim):
@@ -346,10 +360,7 @@ def test_one_key_stands_out_at_every_edge(backend, aim):
     Query 100 as part of a portion and decoded alone; the page border lies at 96."""
     dev, dt = backend
     H, G, D, V, n, BS, i = 4, 2, 16, 8, 101, 32, 100
-    mk, j = {"chunk_in": (dict(chunk=26), 78), "chunk_out": (dict(chunk=26), 77),
-             "window_in": (dict(window=30, keep_first=4), 71), "window_out": (dict(window=30, keep_first=4), 70),
-             "first_in": (dict(window=30, keep_first=4), 3), "first_out": (dict(window=30, keep_first=4), 4),
-             "far": (dict(), 1)}[aim]
+    mk, j = EDGES[aim]
     q, k, v, kc, vc, bt = attention_case(dev, dt, H, G, D, V, n, BS, seed=3, sharp=(i, j))
     want = O.masked_softmax_attention(q, k, v, 1.0, visible(**mk))
     share = (want[i] - v[j].repeat_interleave(H // G, 0)).abs().max()
@@ -358,6 +369,58 @@ def test_one_key_stands_out_at_every_edge(backend, aim):
     kw = dict(chunk=mk.get("chunk", 0), window=mk.get("window", 0), keep_first=mk.get("keep_first", 0))
     for a in (0, 90, i):                                               # whole prompt, a portion, decoded alone
         got = S.masked_attention(qd[a:].contiguous(), H, G, D, V, kc, vc, seg_meta([n - a], [a], [0], dev, bt), 1.0, **kw)
+        close(got[-1], want[i].reshape(-1), dt)
+
+
+MFMA_BACKEND = [pytest.param(("cuda", torch.bfloat16), id="gpu-bf16", marks=GPU)]
+
+
+@pytest.mark.parametrize("backend", MFMA_BACKEND)
+@pytest.mark.parametrize("H,G,D,V", [(4, 2, 64, 64), (3, 1, 128, 64), (18, 2, 64, 128), (2, 2, 128, 128), (1, 1, 64, 64)])
+@pytest.mark.parametrize("mask", range(len(MASKS)))
+def test_masked_attention_on_the_matrix_cores(backend, H, G, D, V, mask):
+    """The sizes the matrix-core kernel takes: tiles of 16 tokens, portions that start inside a tile's
+    span, a chunk border inside a tile, decoding token by token."""
+    dev, dt = backend
+    mk = MASKS[mask]
+    n, BS, scale = 150, 32, 0.25
+    q, k, v, kc, vc, bt, vt = attention_case(dev, dt, H, G, D, V, n, BS, seed=mask + H, with_twin=True)
+    assert S.masked_mfma_ok(H, G, D, V, dt, dev)
+    sink = rnd(H, seed=9) if mask % 2 else None
+    gate = rnd(n, H + 2, seed=10) if mask % 3 else None
+    want = O.masked_softmax_attention(q, k, v, scale, visible(**mk), softcap=mk.get("softcap", 0.0), sink=sink)
+    if gate is not None:
+        want = want * torch.sigmoid(gate[:, 1:H + 1])[:, :, None]
+    kw = dict(softcap=mk.get("softcap", 0.0), chunk=mk.get("chunk", 0), window=mk.get("window", 0),
+              keep_first=mk.get("keep_first", 0), sink=None if sink is None else sink.float().to(dev))
+    gd = None if gate is None else gate.float().to(dev)
+    qd = q.reshape(n, -1).to(dev).to(dt)
+    for cuts in [(n,), (40, 1, 1, 2, 30, 17), (3, 70), (139,) + (1,) * 11]:
+        def run(a, e):
+            sg = seg_meta([e - a], [a], [0], dev, bt)
+            return S.masked_attention(qd[a:e].contiguous(), H, G, D, V, kc, vc, sg, scale,
+                                      gate=None if gd is None else gd[a:e, 1:], vt=vt, **kw)
+        close(in_portions(run, n, cuts), want.reshape(n, -1), dt)
+    # two sequences in one step share nothing: the second one's rows read its own pages
+    sg = seg_meta([5, n - 100], [n - 5, 100], [0, 1], dev, bt + bt)
+    got = S.masked_attention(torch.cat([qd[n - 5:], qd[100:]]).contiguous(), H, G, D, V, kc, vc, sg, scale,
+                             gate=None if gd is None else torch.cat([gd[n - 5:], gd[100:]])[:, 1:], vt=vt, **kw)
+    close(got, torch.cat([want[n - 5:], want[100:]]).reshape(n - 95, -1), dt)
+
+
+@pytest.mark.parametrize("backend", MFMA_BACKEND)
+@pytest.mark.parametrize("aim", ["chunk_in", "chunk_out", "window_in", "window_out", "first_in", "first_out", "far"])
+def test_one_key_stands_out_on_the_matrix_cores(backend, aim):
+    dev, dt = backend
+    H, G, D, V, n, BS, i = 4, 2, 64, 64, 101, 32, 100
+    mk, j = EDGES[aim]
+    q, k, v, kc, vc, bt, vt = attention_case(dev, dt, H, G, D, V, n, BS, seed=3, sharp=(i, j), with_twin=True)
+    want = O.masked_softmax_attention(q, k, v, 1.0, visible(**mk))
+    qd = q.reshape(n, -1).to(dev).to(dt)
+    kw = dict(chunk=mk.get("chunk", 0), window=mk.get("window", 0), keep_first=mk.get("keep_first", 0))
+    for a in (0, 90, i):
+        got = S.masked_attention(qd[a:].contiguous(), H, G, D, V, kc, vc, seg_meta([n - a], [a], [0], dev, bt), 1.0,
+                                 vt=vt, **kw)
         close(got[-1], want[i].reshape(-1), dt)
 
 
@@ -573,6 +636,9 @@ def test_long_decoding_past_windows_and_chunks(backend):
 
 
 OTHER = {
+    "matrix_core_sizes": [(att(heads=4, kv_heads=2, dim=64, vdim=64, chunk=24), 32),
+                          (par(heads=2, kv_heads=1, dim=128, vdim=64, window=20, keep=5, rot=64, mh=2, md=64, mv=64), 0),
+                          (dlt(heads=2, kv_heads=1, dim=64, vdim=128), 16), (att(heads=4, kv_heads=2, dim=64, vdim=64, chunk=24), 0)],
     "one_head_everywhere": [(att(heads=1, kv_heads=1, dim=4, vdim=4), 8), (par(heads=1, kv_heads=1, mh=1), 8),
                             (dlt(heads=1, kv_heads=1), 8)],
     "delta_first_grouped_no_conv": [(dlt(heads=6, kv_heads=2, dim=5, vdim=3, conv=1, ra=1, rg=1), 0), (att(v_mix=False), 8)],
@@ -587,7 +653,8 @@ OTHER = {
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("name", sorted(OTHER))
 def test_other_sizes(backend, name):
-    d = config(OTHER[name], width=40 if name != "wide_taps_unaligned" else 34, eps=1e-3, embed_scale=1.0)
+    d = config(OTHER[name], width={"wide_taps_unaligned": 34, "matrix_core_sizes": 64}.get(name, 40), eps=1e-3,
+               embed_scale=1.0)
     W = weights(d, 11)
     tokens = toks(40, d["vocab"], 12)
     want = O.forward(d, W, tokens)
