@@ -408,10 +408,10 @@ class LizesunModel:
                                 keep_first=a.keep_first, sink=L["sink"], vt=vts[ci])
         xr = x[:, nl:]
         hd, hv = b.heads * b.dim, b.heads * b.vdim
-        o = S.matrix_memory(xr, b.heads, b.dim, b.vdim, L["gate_bias"], b.gate_cap, states[f"mem{j}"],
-                            states[f"memn{j}"], states[f"memm{j}"], inp.seg)
+        o, mul = S.matrix_memory(xr, b.heads, b.dim, b.vdim, L["gate_bias"], b.gate_cap, states[f"mem{j}"],
+                                 states[f"memn{j}"], states[f"memm{j}"], inp.seg, defer_scale=True)
         orr = S.head_norm_gate(o, xr[:, 2 * hd + hv:2 * hd + 2 * hv], L["mem_norm"], b.heads, b.vdim,
-                               self.cfg.norm_eps, self.dtype)
+                               self.cfg.norm_eps, self.dtype, mul=mul)
         return self._lin32(ol, L["wo_l"]), self._lin32(orr, L["wo_r"])
 
     def _delta(self, li: int, h, inp: S.SegStepInputs, states) -> torch.Tensor:

@@ -116,9 +116,9 @@ _SIGS = {
     "k8s_masked_attn_rows": [P, P, P, P, I, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, I, F, F, I, P],
     "k8s_masked_attn_mfma_ok": [I, I, I, I],
     "k8s_masked_attn_mfma": [P, P, P, P, I, P, I, P, P, I, P, I, I, I, I, I, I, I, I, F, F, P],
-    "k8s_gated_delta": [P, I, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, P],
-    "k8s_matrix_memory": [P, I, P, F, P, P, P, P, P, P, P, P, I, I, I, I, I, F, P],
-    "k8s_head_norm_gate": [P, P, I, P, I, P, I, I, I, F, I, P],
+    "k8s_gated_delta": [P, I, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, P, P, I, P, P, P],
+    "k8s_matrix_memory": [P, I, P, F, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P, P, I, P, P, P, P],
+    "k8s_head_norm_gate": [P, P, I, P, I, P, I, I, I, F, I, P, P],
     "k8s_walks": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
 }
 # entry points whose C return type is not int

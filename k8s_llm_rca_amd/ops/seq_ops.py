@@ -739,24 +739,29 @@ def masked_mfma_ok(H: int, G: int, D: int, V: int, dtype, device) -> bool:
 
 
 def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, H: int, V: int, eps: float,
-                   out_dtype) -> torch.Tensor:
-    """``o / rms(o over each head's V) * w * sigmoid(gate)`` of fp32 rows ``o`` [T, H V]; ``w`` [V] (shared by the
-    heads) or [H V]; ``gate`` [T, H V] fp32 (row stride free)."""
+                   out_dtype, mul: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``u / rms(u over each head's V) * w * sigmoid(gate)`` of fp32 rows ``o`` [T, H V], ``u = o * mul`` with ``mul``
+    [T, H] where given; ``w`` [V] (shared by the heads) or [H V]; ``gate`` [T, H V] fp32 (row stride free)."""
     T = o.shape[0]
     out = torch.empty(T, H * V, dtype=out_dtype, device=o.device)
     if use_hip(o):
         assert o.dtype == gate.dtype == w.dtype == torch.float32 and o.is_contiguous() and gate.stride(1) == 1
         assert w.numel() in (V, H * V)
+        assert mul is None or (mul.dtype == torch.float32 and mul.is_contiguous() and mul.numel() == T * H)
         check(lib().k8s_head_norm_gate(ptr(o), ptr(gate), gate.stride(0), ptr(w), V if w.numel() == H * V else 0,
-                                       ptr(out), T, H, V, float(eps), _dt(out_dtype), stream_ptr(o)), "head_norm_gate")
+                                       ptr(out), T, H, V, float(eps), _dt(out_dtype), stream_ptr(o), ptr(mul)),
+              "head_norm_gate")
         return out
     oh = o.view(T, H, V)
+    if mul is not None:
+        oh = oh * mul.view(T, H, 1)
     oh = oh * torch.rsqrt(oh.pow(2).mean(-1, keepdim=True) + eps)
     wv = w.view(H, V) if w.numel() == H * V else w.view(1, V)
     out.copy_((oh * wv * torch.sigmoid(gate[:, :H * V]).view(T, H, V)).reshape(T, H * V).to(out_dtype))
     return out
 
 
+MAT_CHUNK = 64      # rows per chunk of the chunk-parallel matrix-state recurrences
 UNIT_EPS = 1e-6     # q and k of the delta rule: x / sqrt(sum(x^2) + UNIT_EPS)
 
 
@@ -776,10 +781,19 @@ def gated_delta(qkv: torch.Tensor, H: int, G: int, D: int, V: int, a: torch.Tens
         assert beta.dtype == torch.float32 and beta.stride(1) == 1 and beta.shape[1] >= H
         assert rate.dtype == dt_bias.dtype == torch.float32 and rate.numel() == H and dt_bias.numel() == H * D
         assert state.is_contiguous() and state.shape[1:] == (H, D, V)
+        # long portions: chunks in parallel (end states and step-matrix products from zero / identity, a carry
+        # over the chunks, the chunks again from their start states); short ones token by token
+        cr = seg.chunk_ranges(MAT_CHUNK, 2 * MAT_CHUNK)
+        chunks, c0, cs, cx, nch = None, None, None, None, 0
+        if cr is not None:
+            chunks, c0 = cr
+            nch = chunks.shape[0]
+            cs = scratch(nch * H * D * V, torch.float32, qkv.device)
+            cx = scratch(nch * H * D * D, torch.float32, qkv.device)
         check(lib().k8s_gated_delta(ptr(qkv), _dt(qkv.dtype), ptr(a), ptr(rate), ptr(dt_bias), ptr(beta),
                                     beta.stride(0), ptr(state), ptr(seg.seg_row0), ptr(seg.seg_pos0),
                                     ptr(seg.seg_slot), ptr(out), seg.n_seg, T, H, G, D, V, float(UNIT_EPS),
-                                    stream_ptr(qkv)), "gated_delta")
+                                    stream_ptr(qkv), ptr(chunks), nch, ptr(c0), ptr(cs), ptr(cx)), "gated_delta")
         return out
     x = qkv.float()
     q = x[:, :G * D].view(T, G, D)
@@ -807,13 +821,15 @@ DEN_EPS = 1e-6      # matrix memory: o = S^T q / (max(|n.q|, exp(-m)) + DEN_EPS)
 
 
 def matrix_memory(x: torch.Tensor, H: int, D: int, V: int, gate_bias: torch.Tensor, cap: float,
-                  state: torch.Tensor, nstate: torch.Tensor, mstate: torch.Tensor, seg: SegMeta) -> torch.Tensor:
+                  state: torch.Tensor, nstate: torch.Tensor, mstate: torch.Tensor, seg: SegMeta,
+                  defer_scale: bool = False):
     """Matrix memory with exponential gates per head, fp32.  Rows of ``x`` [T, 2 H D + 2 H V + 2 H] fp32 =
     (q | k | v | . | i | f): q is scaled by ``D^(-1/2)``; the log gates are ``i = cap tanh((i + b_i) / cap)`` and
     ``f = logsigmoid(cap tanh((f + b_f) / cap))`` with ``gate_bias`` [2 H] = (b_i | b_f).  With the running maximum
     ``m`` (0 at the start of a sequence):  ``m' = max(f + m, i)``;  ``S <- e^(f + m - m') S + e^(i - m') k v^T``;  n likewise
     with k alone;  ``o = S^T q / (max(|n.q|, e^(-m')) + DEN_EPS)``.  ``state`` [slots, H, D, V], ``nstate`` [slots, H, D],
-    ``mstate`` [slots, H] fp32 are read (past position 0) and advanced.  Returns o [T, H V] fp32."""
+    ``mstate`` [slots, H] fp32 are read (past position 0) and advanced.  Returns o [T, H V] fp32; with
+    ``defer_scale`` (o', mul) with ``o = o' * mul[:, :, None]``, ``mul`` [T, H], for :func:`head_norm_gate` to apply."""
     T = x.shape[0]
     out = torch.empty(T, H * V, dtype=torch.float32, device=x.device)
     if use_hip(x):
@@ -822,11 +838,24 @@ def matrix_memory(x: torch.Tensor, H: int, D: int, V: int, gate_bias: torch.Tens
         assert state.is_contiguous() and state.shape[1:] == (H, D, V) and nstate.is_contiguous()
         assert nstate.shape[1:] == (H, D) and mstate.is_contiguous() and mstate.shape[1:] == (H,)
         ab = scratch(T * H * 3, torch.float32, x.device)
+        nq = scratch(T * H, torch.float32, x.device)
+        mul = scratch((T, H), torch.float32, x.device)
+        # long portions: chunks in parallel (end states from zero, a carry over the chunks, the chunks again
+        # from their start states); short ones token by token
+        cr = seg.chunk_ranges(MAT_CHUNK, 2 * MAT_CHUNK)
+        chunks, c0, cs, cx, cdec, nch = None, None, None, None, None, 0
+        if cr is not None:
+            chunks, c0 = cr
+            nch = chunks.shape[0]
+            cs = scratch(nch * H * D * V, torch.float32, x.device)
+            cx = scratch(nch * H * D, torch.float32, x.device)
+            cdec = scratch(nch * H, torch.float32, x.device)
         check(lib().k8s_matrix_memory(ptr(x), x.stride(0), ptr(gate_bias), float(cap), ptr(state), ptr(nstate),
                                       ptr(mstate), ptr(seg.seg_row0), ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(ab),
-                                      ptr(out), seg.n_seg, T, H, D, V, float(DEN_EPS), stream_ptr(x)),
-              "matrix_memory")
-        return out
+                                      ptr(nq), ptr(mul), ptr(out), seg.n_seg, T, H, D, V, float(DEN_EPS),
+                                      0 if defer_scale else 1, stream_ptr(x), ptr(chunks), nch, ptr(c0), ptr(cs),
+                                      ptr(cx), ptr(cdec)), "matrix_memory")
+        return (out, mul) if defer_scale else out
     HD, HV = H * D, H * V
     q = x[:, :HD].view(T, H, D) * D ** -0.5
     k = x[:, HD:2 * HD].view(T, H, D)
@@ -850,4 +879,4 @@ def matrix_memory(x: torch.Tensor, H: int, D: int, V: int, gate_bias: torch.Tens
             den = torch.maximum((n * q[r]).sum(-1).abs(), torch.exp(-m)) + DEN_EPS
             out[r] = (torch.einsum("hdv,hd->hv", S, q[r]) / den[:, None]).reshape(-1)
         state[sl], nstate[sl], mstate[sl] = S, n, m
-    return out
+    return (out, None) if defer_scale else out

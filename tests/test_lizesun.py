@@ -442,9 +442,10 @@ def test_sink_takes_its_share(backend):
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("H,G,D,V", [(4, 2, 8, 12), (2, 2, 6, 4), (3, 1, 33, 70), (1, 1, 128, 64), (2, 1, 200, 5)])
-def test_gated_delta_across_portions_and_slots(backend, H, G, D, V):
+@pytest.mark.parametrize("T", [41, 333])
+def test_gated_delta_across_portions_and_slots(backend, H, G, D, V, T):
+    """T = 333: portions of more than 128 rows run in chunks of 64 in parallel (on the device)."""
     dev, dt = backend
-    T = 41
     x = rnd(T, 2 * G * D + H * V, seed=D).to(torch.bfloat16).double()
     a, beta = rnd(T, H * D, seed=2), rnd(T, H + 3, seed=3, std=2.0)
     rate, bias = torch.exp(rnd(H, seed=4, std=0.5)), rnd(H * D, seed=5) - 0.5
@@ -466,7 +467,7 @@ def test_gated_delta_across_portions_and_slots(backend, H, G, D, V):
             want[i, h] = Sh.T @ qq
     f32 = lambda z: z.float().to(dev)  # noqa: E731
     xd, bd = x.to(dev).to(dt), f32(beta)
-    for cuts in [(T,), (1, 1, 2, 17, 3), (16, 16, 1)]:
+    for cuts in [(T,), (1, 1, 2, 17, 3), (16, 16, 1)] if T < 100 else [(T,), (200, 133), (130, 1, 1, 201)]:
         state = torch.full((3, H, D, V), float("nan"), device=dev)
 
         def run(s, e):
@@ -478,9 +479,11 @@ def test_gated_delta_across_portions_and_slots(backend, H, G, D, V):
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("H,D,V", [(3, 8, 12), (1, 4, 4), (2, 33, 70), (2, 128, 64), (1, 200, 130)])
-def test_matrix_memory_across_portions_and_slots(backend, H, D, V):
+@pytest.mark.parametrize("T", [41, 333])
+def test_matrix_memory_across_portions_and_slots(backend, H, D, V, T):
+    """T = 333: portions of more than 128 rows run in chunks of 64 in parallel (on the device)."""
     dev, dt = backend
-    T, cap = 41, 5.0
+    cap = 5.0
     x = rnd(T, 2 * H * D + 2 * H * V + 2 * H, seed=D)
     x[:, -2 * H:] *= 4.0                                                # gates that reach the cap
     gb = rnd(2 * H, seed=2)
@@ -494,12 +497,16 @@ def test_matrix_memory_across_portions_and_slots(backend, H, D, V):
     want = O.matrix_memory(x, t, "", {"heads": H, "dim": D, "vdim": V, "gate_cap": cap}, 1e-5)
     f32 = lambda z: z.float().to(dev)  # noqa: E731
     xd, ones, zero = f32(x), torch.ones(HV, device=dev), torch.zeros(T, HV, device=dev)
-    for cuts in [(T,), (1, 1, 2, 17, 3), (16, 16, 1)]:
+    for k, cuts in enumerate([(T,), (1, 1, 2, 17, 3), (16, 16, 1)] if T < 100 else [(T,), (200, 133), (130, 1, 1, 201)]):
         st = [torch.full((3,) + s, float("nan"), device=dev) for s in ((H, D, V), (H, D), (H,))]
 
         def run(s, e):
-            o = S.matrix_memory(xd[s:e], H, D, V, f32(gb), cap, *st, seg_meta([e - s], [s], [2], dev))
-            return S.head_norm_gate(o, zero[s:e], ones, H, V, 1e-5, torch.float32)
+            sg = seg_meta([e - s], [s], [2], dev)
+            if k % 2:        # the scale applied by the op itself, or handed on to the norm
+                o, mul = S.matrix_memory(xd[s:e], H, D, V, f32(gb), cap, *st, sg), None
+            else:
+                o, mul = S.matrix_memory(xd[s:e], H, D, V, f32(gb), cap, *st, sg, defer_scale=True)
+            return S.head_norm_gate(o, zero[s:e], ones, H, V, 1e-5, torch.float32, mul=mul)
         close(in_portions(run, T, cuts), want, torch.float32, scale=3.0)
 
 
@@ -531,6 +538,40 @@ def test_two_sequences_in_one_step_keep_their_own_state(backend):
     o2 = S.matrix_memory(f32(torch.cat([xb[1:], xa[5:]])), H, D, V, f32(gb), cap, *st, seg_meta([5, 4], [1, 5], [0, 3], dev))
     close(torch.cat([o1[:5], o2[5:]]), alone(xa), torch.float32)
     close(torch.cat([o1[5:], o2[:5]]), alone(xb), torch.float32)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_long_and_short_portions_in_one_step(backend):
+    """A portion long enough for the chunk-parallel kernels beside a short one and a single token: every
+    sequence's result is what it gets alone."""
+    dev, dt = backend
+    H, G, D, V = 2, 1, 16, 24
+    lens, pos0, slots = [200, 3, 1], [0, 5, 9], [2, 0, 1]
+    T = sum(lens)
+    x = rnd(T, 2 * G * D + H * V, seed=1).to(torch.bfloat16).double()
+    a, beta = rnd(T, H * D, seed=2), rnd(T, H, seed=3)
+    rate, bias = torch.exp(rnd(H, seed=4, std=0.5)), rnd(H * D, seed=5) - 0.5
+    xm, gb = rnd(T, 2 * H * (D + V) + 2 * H, seed=6), rnd(2 * H, seed=7)
+    f32 = lambda z: z.float().to(dev)  # noqa: E731
+
+    def states(fill):
+        return [torch.full((3,) + s, fill, device=dev) for s in ((H, D, V), (H, D, V), (H, D), (H,))]
+
+    def run(st, xs, as_, bs, xms, sg):
+        o1 = S.gated_delta(xs.to(dev).to(dt).contiguous(), H, G, D, V, f32(as_), f32(rate), f32(bias), f32(bs), st[0], sg)
+        o2 = S.matrix_memory(f32(xms), H, D, V, f32(gb), 4.0, st[1], st[2], st[3], sg)
+        return o1, o2
+    together = states(0.25)                    # the two continuing sequences start from some state
+    o1, o2 = run(together, x, a, beta, xm, seg_meta(lens, pos0, slots, dev))
+    at = 0
+    for n, p0, sl in zip(lens, pos0, slots):
+        alone = states(0.25)
+        w1, w2 = run(alone, x[at:at + n], a[at:at + n], beta[at:at + n], xm[at:at + n], seg_meta([n], [p0], [sl], dev))
+        close(o1[at:at + n], w1, torch.float32, scale=5.0)
+        close(o2[at:at + n], w2, torch.float32, scale=5.0)
+        for u, v in zip(together, alone):
+            close(u[sl], v[sl], torch.float32, scale=5.0)
+        at += n
 
 
 # ------------------------------------------------------------------ whole models
@@ -614,6 +655,18 @@ def test_edges_and_page_borders_with_sharp_scores(backend):
     tokens = toks(100, d["vocab"], 7)
     want = O.forward(d, W, tokens)
     for cuts in [(100,), (23, 2, 24, 15, 2, 30), (47,)]:
+        eng = engine(d, W, backend)
+        assert agrees(feed_all(eng, eng.new_sequence(), tokens, cuts), want, backend[1], mult=2.0), cuts
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_long_portions_then_decoding(backend):
+    """Portions long enough for the chunk-parallel recurrences, cut off a chunk's border, then single tokens."""
+    d = default_config()
+    W = weights(d, 17)
+    tokens = toks(330, d["vocab"], 18)
+    want = O.forward(d, W, tokens)
+    for cuts in [(321,), (150, 171)]:
         eng = engine(d, W, backend)
         assert agrees(feed_all(eng, eng.new_sequence(), tokens, cuts), want, backend[1], mult=2.0), cuts
 
