@@ -303,8 +303,13 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
     for (int dt = 0; dt < NV; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const float sc2 = a.scale * kLog2e, cap2 = a.softcap * kLog2e, icap = a.softcap > 0.f ? a.scale / a.softcap : 0.f;
+  // a block whose 32 keys every query of a full tile sees needs no mask: all keys at or before the first
+  // position, inside the last query's chunk, and inside the last query's window or among the kept tokens
+  const int cl_lo = a.chunk > 0 ? (pos_last / a.chunk) * a.chunk : 0;
+  const int wl_lo = a.window > 0 ? pos_last - a.window + 1 : 0;
   for (int bi = 0; bi < nblk; ++bi) {
     const int kb = bi < nblkA ? a_beg + 32 * bi : lo_al + 32 * (bi - nblkA);
+    const bool open_blk = ntok == 16 && kb + 31 <= pos0 && kb >= cl_lo && (kb >= wl_lo || kb + 32 <= keep);
     const int page = pages[kb / a.BS], off = kb % a.BS;
     const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK;
     bf16x8 kf[2][NDC];
@@ -336,7 +341,7 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int key = kb + 8 * hq + 4 * t + i;
-            const bool ok = qvalid && key <= posq && key >= cq_lo && (key >= wq_lo || key < keep);
+            const bool ok = open_blk || (qvalid && key <= posq && key >= cq_lo && (key >= wq_lo || key < keep));
             float s2;
             if (a.softcap > 0.f) {
               // cap tanh(x), tanh(x) = 1 - 2 / (1 + e^(2x)), in log2 units
@@ -353,9 +358,11 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
         for (int j = 1; j < 8; ++j) cmax = fmaxf(cmax, p[j]);
         cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
         cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
-        const float mn = fmaxf(m2[hh], cmax);
+        // the maximum moves only where a query meets a larger score; while no query of the wave does, the
+        // accumulators need no rescaling (a wave-uniform branch)
+        const bool grow = cmax > m2[hh];
+        const float mn = grow ? cmax : m2[hh];
         const float ms = mn == -INFINITY ? 0.f : mn;       // a query that has seen no key yet
-        const float alpha = __builtin_amdgcn_exp2f(m2[hh] - ms);
         float ps = 0.f;
         bf16x8 pf;
 #pragma unroll
@@ -364,17 +371,21 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
           ps += e;
           pf[j] = (__bf16)e;
         }
-        l[hh] = l[hh] * alpha + ps;
-        m2[hh] = mn;
-        float ai[4];
+        if (__any(grow)) {
+          const float alpha = __builtin_amdgcn_exp2f(m2[hh] - ms);
+          l[hh] *= alpha;
+          m2[hh] = mn;
+          float ai[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ai[i] = __shfl(alpha, 4 * hq + i, 64);
+          for (int i = 0; i < 4; ++i) ai[i] = __shfl(alpha, 4 * hq + i, 64);
 #pragma unroll
-        for (int dt = 0; dt < NV; ++dt) {
+          for (int dt = 0; dt < NV; ++dt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) o[hh][dt][i] *= ai[i];
-          o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[dt], o[hh][dt], 0, 0, 0);
+            for (int i = 0; i < 4; ++i) o[hh][dt][i] *= ai[i];
         }
+        l[hh] += ps;
+#pragma unroll
+        for (int dt = 0; dt < NV; ++dt) o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[dt], o[hh][dt], 0, 0, 0);
       }
     }
   }

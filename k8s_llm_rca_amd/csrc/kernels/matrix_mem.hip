@@ -147,7 +147,9 @@ struct MatArgs {
   float* cdec;         // [chunks][H] (memory)
 };
 
-template <int DPT, int KIND, int MODE, typename TA>
+// FULL: D == 4 * DPT, every thread's DPT rows exist (no guards in the token loop: its LDS reads become
+// 16-byte ones)
+template <int DPT, int KIND, int MODE, bool FULL, typename TA>
 __global__ void __launch_bounds__(256) matrix_state_kernel(MatArgs p) {
   extern __shared__ float sm[];
   const int it = blockIdx.x, hh = blockIdx.y, c0 = blockIdx.z * kMemVb, tid = threadIdx.x;
@@ -261,7 +263,7 @@ __global__ void __launch_bounds__(256) matrix_state_kernel(MatArgs p) {
 #pragma unroll
         for (int i = 0; i < DPT; ++i) {
           const int d = dg * DPT + i;
-          if (d < D) {
+          if (FULL || d < D) {
             S[i] *= gd[d];
             ks = fmaf(S[i], kq[d], ks);
           }
@@ -272,7 +274,7 @@ __global__ void __launch_bounds__(256) matrix_state_kernel(MatArgs p) {
 #pragma unroll
         for (int i = 0; i < DPT; ++i) {
           const int d = dg * DPT + i;
-          if (d < D) {
+          if (FULL || d < D) {
             S[i] = fmaf(kq[d], u, S[i]);
             if (MODE != 1) acc = fmaf(S[i], qq[d], acc);
           }
@@ -284,7 +286,7 @@ __global__ void __launch_bounds__(256) matrix_state_kernel(MatArgs p) {
 #pragma unroll
         for (int i = 0; i < DPT; ++i) {
           const int d = dg * DPT + i;
-          if (d < D) {
+          if (FULL || d < D) {
             S[i] = fmaf(fa, S[i], kq[d] * iv);
             if (MODE != 1) acc = fmaf(S[i], qq[d], acc);
           }
@@ -340,8 +342,9 @@ __global__ void __launch_bounds__(256) delta_carry_kernel(MatArgs p, const int* 
   extern __shared__ float sm[];
   const int sg = blockIdx.x, hh = blockIdx.y, c0 = blockIdx.z * kMemVb, tid = threadIdx.x;
   const int H = p.H, D = p.D, V = p.V;
+  constexpr int DP = 4 * DPT;     // row length of the transposed product in LDS (>= D)
   float* sS = sm;                 // [D][64]
-  float* sP = sS + D * kMemVb;    // [D][D]
+  float* sP = sS + D * kMemVb;    // [D][DP]
   const int dg = tid & 3, vl = tid >> 2, c = c0 + vl;
   const bool cown = c < V;
   float* st = p.state + ((size_t)p.seg_slot[sg] * H + hh) * D * V + c;
@@ -361,19 +364,26 @@ __global__ void __launch_bounds__(256) delta_carry_kernel(MatArgs p, const int* 
       const int d = dg * DPT + i;
       if (d < D) sS[d * kMemVb + vl] = S[i];
     }
-    for (int e = tid; e < D * D; e += 256) sP[e] = P[e];
+    for (int e = tid; e < D * D; e += 256) {            // transposed: sP[j][d], a thread's DPT rows side by side
+      const int d = e / D, j = e - d * D;
+      sP[j * DP + d] = P[e];
+    }
     __syncthreads();
+    float acc[DPT];
 #pragma unroll
     for (int i = 0; i < DPT; ++i) {
       const int d = dg * DPT + i;
-      if (d < D) {
-        float acc = cown ? ck[(size_t)d * V] : 0.f;     // the chunk's end state from zero
-        if (cown) ck[(size_t)d * V] = S[i];             // becomes its start state
-        const float* pr = sP + d * D;
-        for (int j = 0; j < D; ++j) acc = fmaf(pr[j], sS[j * kMemVb + vl], acc);
-        S[i] = acc;
-      }
+      acc[i] = (cown && d < D) ? ck[(size_t)d * V] : 0.f;   // the chunk's end state from zero
+      if (cown && d < D) ck[(size_t)d * V] = S[i];          // becomes its start state
     }
+    for (int j = 0; j < D; ++j) {
+      const float sj = sS[j * kMemVb + vl];
+      const float* pc = sP + j * DP + dg * DPT;
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) acc[i] = fmaf(pc[i], sj, acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) S[i] = acc[i];
   }
 #pragma unroll
   for (int i = 0; i < DPT; ++i) {
@@ -403,13 +413,19 @@ __global__ void __launch_bounds__(256) head_norm_sigmoid_kernel(const float* __r
   for (int c = lane; c < V; c += 64) stx(out, (size_t)rh * V + c, op[c] * rn * wp[c] * sigmoid_f(g[c]));
 }
 
-template <int DPT, int KIND, int MODE, typename TA>
-static int launch_state_mode(const MatArgs& p, int items, int cols, size_t lds, hipStream_t s) {
-  auto k = matrix_state_kernel<DPT, KIND, MODE, TA>;
+template <int DPT, int KIND, int MODE, bool FULL, typename TA>
+static int launch_state_full(const MatArgs& p, int items, int cols, size_t lds, hipStream_t s) {
+  auto k = matrix_state_kernel<DPT, KIND, MODE, FULL, TA>;
   if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
     return (int)hipGetLastError();
   hipLaunchKernelGGL(k, dim3(items, p.H, (cols + kMemVb - 1) / kMemVb), dim3(256), lds, s, p);
   return (int)hipGetLastError();
+}
+
+template <int DPT, int KIND, int MODE, typename TA>
+static int launch_state_mode(const MatArgs& p, int items, int cols, size_t lds, hipStream_t s) {
+  return p.D == 4 * DPT ? launch_state_full<DPT, KIND, MODE, true, TA>(p, items, cols, lds, s)
+                        : launch_state_full<DPT, KIND, MODE, false, TA>(p, items, cols, lds, s);
 }
 
 // n_chunks == 0: every segment token by token; otherwise the two chunk passes around the carry
@@ -417,13 +433,15 @@ template <int DPT, int KIND, typename TA>
 static int launch_state_dpt(const MatArgs& p, int n_seg, int n_chunks, const int* seg_chunk0, hipStream_t s) {
   const int D = p.D, V = p.V;
   const size_t lds = (size_t)(kMemTb * ((KIND == 0 ? 3 : 2) * D + kMemVb + 4)) * sizeof(float);
-  if (n_chunks <= 0) return launch_state_mode<DPT, KIND, 0, TA>(p, n_seg, V + (KIND == 1 ? 1 : 0), lds, s);
+  // (the delta rule's carry holds a D x D product and D x 64 state entries in LDS: token by token where that does not fit)
+  const size_t cl = (size_t)(D * kMemVb + D * 4 * DPT) * sizeof(float);
+  if (n_chunks <= 0 || (KIND == 0 && cl > 160 * 1024))
+    return launch_state_mode<DPT, KIND, 0, TA>(p, n_seg, V + (KIND == 1 ? 1 : 0), lds, s);
   int rc = launch_state_mode<DPT, KIND, 1, TA>(p, n_chunks, V + (KIND == 1 ? 1 : D), lds, s);
   if (rc) return rc;
   if (KIND == 1) {
     hipLaunchKernelGGL(memory_carry_kernel, dim3(n_seg, p.H, (D * V + D + 255) / 256), dim3(256), 0, s, p, seg_chunk0);
   } else {
-    const size_t cl = (size_t)(D * kMemVb + D * D) * sizeof(float);
     auto k = delta_carry_kernel<DPT>;
     if (cl > 48 * 1024 && hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)cl))
       return (int)hipGetLastError();

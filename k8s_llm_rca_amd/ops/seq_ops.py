@@ -762,6 +762,15 @@ def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, H: int,
 
 
 MAT_CHUNK = 64      # rows per chunk of the chunk-parallel matrix-state recurrences
+MAT_FILL_GROUPS = 1024   # workgroups (segments x heads x 64-column blocks) from which token by token fills the chip
+
+
+def _mat_chunks(seg: SegMeta, H: int, V: int):
+    """The chunk ranges of a step for the matrix-state recurrences, or None where they run token by token:
+    no long portion, or enough sequences that the sequential form fills the chip at less than half the work."""
+    if seg.n_seg * H * -(-V // 64) >= MAT_FILL_GROUPS:
+        return None
+    return seg.chunk_ranges(MAT_CHUNK, 2 * MAT_CHUNK)
 UNIT_EPS = 1e-6     # q and k of the delta rule: x / sqrt(sum(x^2) + UNIT_EPS)
 
 
@@ -783,7 +792,7 @@ def gated_delta(qkv: torch.Tensor, H: int, G: int, D: int, V: int, a: torch.Tens
         assert state.is_contiguous() and state.shape[1:] == (H, D, V)
         # long portions: chunks in parallel (end states and step-matrix products from zero / identity, a carry
         # over the chunks, the chunks again from their start states); short ones token by token
-        cr = seg.chunk_ranges(MAT_CHUNK, 2 * MAT_CHUNK)
+        cr = _mat_chunks(seg, H, V)
         chunks, c0, cs, cx, nch = None, None, None, None, 0
         if cr is not None:
             chunks, c0 = cr
@@ -842,7 +851,7 @@ def matrix_memory(x: torch.Tensor, H: int, D: int, V: int, gate_bias: torch.Tens
         mul = scratch((T, H), torch.float32, x.device)
         # long portions: chunks in parallel (end states from zero, a carry over the chunks, the chunks again
         # from their start states); short ones token by token
-        cr = seg.chunk_ranges(MAT_CHUNK, 2 * MAT_CHUNK)
+        cr = _mat_chunks(seg, H, V)
         chunks, c0, cs, cx, cdec, nch = None, None, None, None, None, 0
         if cr is not None:
             chunks, c0 = cr

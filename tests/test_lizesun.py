@@ -507,7 +507,7 @@ def test_matrix_memory_across_portions_and_slots(backend, H, D, V, T):
             else:
                 o, mul = S.matrix_memory(xd[s:e], H, D, V, f32(gb), cap, *st, sg, defer_scale=True)
             return S.head_norm_gate(o, zero[s:e], ones, H, V, 1e-5, torch.float32, mul=mul)
-        close(in_portions(run, T, cuts), want, torch.float32, scale=3.0)
+        close(in_portions(run, T, cuts), want, torch.float32, scale=3.0 if T < 100 else 6.0)
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
