@@ -249,6 +249,7 @@ struct MaskArgs {
   const int* bt;
   int maxb;
   const int* items;       // [n][4]: segment, first row, tokens (<= 16), position of the first token
+  int n_items;
   const float* sink;      // [H] or null
   const float* gate;      // [T] rows of stride gs, column h, or null
   int gs;
@@ -259,13 +260,15 @@ struct MaskArgs {
 
 __device__ __forceinline__ bf16x8 mld16(const uint16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
-template <int NDC, int NV, int HW>
+template <int NDC, int NV, int HW, bool CAP>
 __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   constexpr int D = NDC * 32, V = NV * 16;
   constexpr float kLog2e = 1.4426950408889634f;
   const int lane = threadIdx.x & 63, r = lane & 15, hq = lane >> 4;
   const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int item = blockIdx.x;
+  // tiles are listed by position within their segments and a later tile mostly has more keys: the
+  // last ones start first, so the launch does not end on its longest items
+  const int item = a.n_items - 1 - blockIdx.x;
   const int sg = a.items[item * 4], row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2],
             pos0 = a.items[item * 4 + 3];
   const int H = a.H, hpg = H / a.G, NK = a.G * D, NVt = a.G * V;
@@ -307,87 +310,124 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   // position, inside the last query's chunk, and inside the last query's window or among the kept tokens
   const int cl_lo = a.chunk > 0 ? (pos_last / a.chunk) * a.chunk : 0;
   const int wl_lo = a.window > 0 ? pos_last - a.window + 1 : 0;
+  // The wave's heads share one key / value head (the launch picks HW so).  A block's page lookup, key
+  // loads and value loads are dependent memory accesses, so they are issued a block ahead into the SAME
+  // registers: the next keys as soon as this block's scores are formed, the next values as soon as this
+  // block's value products are issued; the softmax and the products run meanwhile.
+  const int g = h0 / hpg;
+  bf16x8 kf[2][NDC];
+  bf16x8 vf[NV];
+  auto block_at = [&](int bi) { return bi < nblkA ? a_beg + 32 * bi : lo_al + 32 * (bi - nblkA); };
+  // lane i of (kbv, pgv, ofv) holds the first key, the page and the offset within the page of block
+  // pg_base + i (64 blocks per fill): the divisions and the page lookup are done for 64 blocks at once,
+  // off the chain of dependent loads
+  int pg_base = 0, kbv = 0, pgv = 0, ofv = 0;
+  auto fill_pages = [&](int base) {
+    pg_base = base;
+    const int bi = base + lane;
+    kbv = block_at(bi);
+    const int pi = kbv / a.BS;
+    ofv = kbv - pi * a.BS;
+    pgv = bi < nblk ? pages[pi] : 0;
+  };
+  fill_pages(0);
+  auto load_k = [&](int page, int off) {
+    const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK + g * D + 8 * hq;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key = 8 * (r >> 2) + 4 * t + (r & 3);
+#pragma unroll
+      for (int cc = 0; cc < NDC; ++cc) kf[t][cc] = mld16(kp + (size_t)key * NK + 32 * cc);
+    }
+  };
+  auto load_v = [&](int page, int off) {
+    const uint16_t* vp = a.vt + ((size_t)page * NVt + (size_t)g * V) * a.BS + off + 8 * hq;
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) vf[dt] = mld16(vp + (size_t)(16 * dt + r) * a.BS);
+  };
+  int kb_next = __shfl(kbv, 0, 64), pg_next = __shfl(pgv, 0, 64), of_next = __shfl(ofv, 0, 64);
+  load_k(pg_next, of_next);
+  load_v(pg_next, of_next);
   for (int bi = 0; bi < nblk; ++bi) {
-    const int kb = bi < nblkA ? a_beg + 32 * bi : lo_al + 32 * (bi - nblkA);
+    const int kb = kb_next;
+    if (bi + 1 < nblk) {
+      if (bi + 1 - pg_base == 64) fill_pages(bi + 1);
+      kb_next = __shfl(kbv, bi + 1 - pg_base, 64);
+      pg_next = __shfl(pgv, bi + 1 - pg_base, 64);
+      of_next = __shfl(ofv, bi + 1 - pg_base, 64);
+    }
     const bool open_blk = ntok == 16 && kb + 31 <= pos0 && kb >= cl_lo && (kb >= wl_lo || kb + 32 <= keep);
-    const int page = pages[kb / a.BS], off = kb % a.BS;
-    const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK;
-    bf16x8 kf[2][NDC];
-    bf16x8 vf[NV];
-    int gprev = -1;
+    float p[HW][8];
 #pragma unroll
     for (int hh = 0; hh < HW; ++hh) {
-      if (hh < nh) {
-        const int g = (h0 + hh) / hpg;
-        if (g != gprev) {
 #pragma unroll
-          for (int t = 0; t < 2; ++t) {
-            const int key = 8 * (r >> 2) + 4 * t + (r & 3);
+      for (int t = 0; t < 2; ++t) {
+        f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int cc = 0; cc < NDC; ++cc) kf[t][cc] = mld16(kp + (size_t)key * NK + g * D + 32 * cc + 8 * hq);
-          }
-          const uint16_t* vp = a.vt + ((size_t)page * NVt + (size_t)g * V) * a.BS + off + 8 * hq;
+        for (int cc = 0; cc < NDC; ++cc)
+          sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][cc], qf[hh][cc], sacc, 0, 0, 0);
 #pragma unroll
-          for (int dt = 0; dt < NV; ++dt) vf[dt] = mld16(vp + (size_t)(16 * dt + r) * a.BS);
-          gprev = g;
-        }
-        float p[8];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int cc = 0; cc < NDC; ++cc)
-            sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][cc], qf[hh][cc], sacc, 0, 0, 0);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int key = kb + 8 * hq + 4 * t + i;
-            const bool ok = open_blk || (qvalid && key <= posq && key >= cq_lo && (key >= wq_lo || key < keep));
-            float s2;
-            if (a.softcap > 0.f) {
-              // cap tanh(x), tanh(x) = 1 - 2 / (1 + e^(2x)), in log2 units
-              const float e = __builtin_amdgcn_exp2f(fminf(sacc[i] * icap * (2.f * kLog2e), 60.f));
-              s2 = cap2 * (1.f - 2.f / (1.f + e));
-            } else {
-              s2 = sacc[i] * sc2;
-            }
-            p[4 * t + i] = ok ? s2 : -INFINITY;
-          }
-        }
-        float cmax = p[0];
-#pragma unroll
-        for (int j = 1; j < 8; ++j) cmax = fmaxf(cmax, p[j]);
-        cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
-        cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
-        // the maximum moves only where a query meets a larger score; while no query of the wave does, the
-        // accumulators need no rescaling (a wave-uniform branch)
-        const bool grow = cmax > m2[hh];
-        const float mn = grow ? cmax : m2[hh];
-        const float ms = mn == -INFINITY ? 0.f : mn;       // a query that has seen no key yet
-        float ps = 0.f;
-        bf16x8 pf;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float e = __builtin_amdgcn_exp2f(p[j] - ms);
-          ps += e;
-          pf[j] = (__bf16)e;
-        }
-        if (__any(grow)) {
-          const float alpha = __builtin_amdgcn_exp2f(m2[hh] - ms);
-          l[hh] *= alpha;
-          m2[hh] = mn;
-          float ai[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) ai[i] = __shfl(alpha, 4 * hq + i, 64);
-#pragma unroll
-          for (int dt = 0; dt < NV; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) o[hh][dt][i] *= ai[i];
-        }
-        l[hh] += ps;
-#pragma unroll
-        for (int dt = 0; dt < NV; ++dt) o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[dt], o[hh][dt], 0, 0, 0);
+        for (int i = 0; i < 4; ++i) p[hh][4 * t + i] = sacc[i];
       }
     }
+    if (bi + 1 < nblk) load_k(pg_next, of_next);
+    bf16x8 pf[HW];
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (CAP) {
+          // cap tanh(x), tanh(x) = 1 - 2 / (1 + e^(2x)), in log2 units
+          const float e = __builtin_amdgcn_exp2f(fminf(p[hh][j] * icap * (2.f * kLog2e), 60.f));
+          p[hh][j] = cap2 * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e));
+        } else {
+          p[hh][j] *= sc2;
+        }
+      }
+      if (!open_blk) {                                     // (a wave-uniform branch)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = kb + 8 * hq + j;                 // j = 4 t + i
+          const bool ok = qvalid && key <= posq && key >= cq_lo && (key >= wq_lo || key < keep);
+          p[hh][j] = ok ? p[hh][j] : -INFINITY;
+        }
+      }
+      float cmax = p[hh][0];
+#pragma unroll
+      for (int j = 1; j < 8; ++j) cmax = fmaxf(cmax, p[hh][j]);
+      cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
+      cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+      // the maximum moves only where a query meets a larger score; while no query of the wave does, the
+      // accumulators need no rescaling (a wave-uniform branch)
+      const bool grow = cmax > m2[hh];
+      const float mn = grow ? cmax : m2[hh];
+      const float ms = mn == -INFINITY ? 0.f : mn;         // a query that has seen no key yet
+      float ps = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float e = __builtin_amdgcn_exp2f(p[hh][j] - ms);
+        ps += e;
+        pf[hh][j] = (__bf16)e;
+      }
+      if (__any(grow)) {
+        const float alpha = __builtin_amdgcn_exp2f(m2[hh] - ms);
+        l[hh] *= alpha;
+        m2[hh] = mn;
+        float ai[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ai[i] = __shfl(alpha, 4 * hq + i, 64);
+#pragma unroll
+        for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[hh][dt][i] *= ai[i];
+      }
+      l[hh] += ps;
+    }
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh)
+#pragma unroll
+      for (int dt = 0; dt < NV; ++dt) o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[hh], vf[dt], o[hh][dt], 0, 0, 0);
+    if (bi + 1 < nblk) load_v(pg_next, of_next);
   }
 #pragma unroll
   for (int hh = 0; hh < HW; ++hh) {
@@ -412,13 +452,21 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   }
 }
 
+template <int NDC, int NV, int HW>
+static int launch_mask_hw(const MaskArgs& a, int n_items, hipStream_t s) {
+  const int waves_all = (a.H + HW - 1) / HW;               // HW heads per wave, up to eight waves per workgroup
+  const int gy = (waves_all + 7) / 8, waves = gy > 1 ? 8 : waves_all;
+  if (a.softcap > 0.f)
+    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, true>), dim3(n_items, gy), dim3(64 * waves), 0, s, a);
+  else
+    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, false>), dim3(n_items, gy), dim3(64 * waves), 0, s, a);
+  return (int)hipGetLastError();
+}
+
+// two heads per wave where the heads of a key / value head come in pairs, else one
 template <int NDC, int NV>
 static int launch_mask_mfma(const MaskArgs& a, int n_items, hipStream_t s) {
-  constexpr int HW = 2;
-  const int waves_all = (a.H + HW - 1) / HW;               // two heads per wave, up to eight waves per workgroup
-  const int gy = (waves_all + 7) / 8, waves = gy > 1 ? 8 : waves_all;
-  hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW>), dim3(n_items, gy), dim3(64 * waves), 0, s, a);
-  return (int)hipGetLastError();
+  return (a.H / a.G) % 2 == 0 ? launch_mask_hw<NDC, NV, 2>(a, n_items, s) : launch_mask_hw<NDC, NV, 1>(a, n_items, s);
 }
 
 }  // namespace k8s
@@ -484,6 +532,7 @@ K8S_API int k8s_masked_attn_mfma(const void* q, const void* kc, const void* vt, 
   a.bt = block_tables;
   a.maxb = maxb;
   a.items = items;
+  a.n_items = n_items;
   a.sink = sink;
   a.gate = gate;
   a.gs = gs;
