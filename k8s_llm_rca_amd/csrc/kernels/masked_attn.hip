@@ -256,11 +256,18 @@ struct MaskArgs {
   uint16_t* out;          // [T][H * V]
   int H, G, BS, chunk, window, keep_first;
   float scale, softcap;
+  // steps of few rows: a tile's key blocks are split over grid.z workgroups, part_blocks blocks each
+  int part_blocks, n_parts;
+  float* pml;             // [items][parts][H][16][2]: a part's maximum (log2 units) and denominator
+  float* po;              // [items][parts][16][H * V]: a part's unnormalised output
 };
 
 __device__ __forceinline__ bf16x8 mld16(const uint16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
-template <int NDC, int NV, int HW, bool CAP>
+// SPLIT: workgroup z walks the blocks [z part_blocks, (z + 1) part_blocks) of its tile and leaves its maximum,
+// denominator and unnormalised output; masked_attn_merge_kernel joins the parts (and adds the sink).  Part
+// borders count blocks of the tile's own block list, so they depend on positions only.
+template <int NDC, int NV, int HW, bool CAP, bool SPLIT>
 __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   constexpr int D = NDC * 32, V = NV * 16;
   constexpr float kLog2e = 1.4426950408889634f;
@@ -286,6 +293,17 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   const int a_end = a.window > 0 ? min(lo_al, (a.keep_first + 31) & ~31) : a_beg;
   const int nblkA = max(0, (a_end - a_beg) >> 5), nblk = nblkA + ((pos_last - lo_al) >> 5) + 1;
   const int* pages = a.bt + (size_t)sg * a.maxb;
+  const int b_lo = SPLIT ? (int)blockIdx.z * a.part_blocks : 0;
+  const int b_hi = (!SPLIT || (int)blockIdx.z == a.n_parts - 1) ? nblk : min(nblk, b_lo + a.part_blocks);
+  if (SPLIT && b_lo >= b_hi) {                             // a part without blocks: nothing to join
+    if (hq == 0)
+      for (int hh = 0; hh < nh; ++hh) {
+        float* ml = a.pml + ((((size_t)item * a.n_parts + blockIdx.z) * H + h0 + hh) * 16 + r) * 2;
+        ml[0] = -INFINITY;
+        ml[1] = 0.f;
+      }
+    return;
+  }
   bf16x8 qf[HW][NDC];
   float m2[HW], l[HW];
   f32x4 o[HW][NV];
@@ -300,7 +318,7 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) qf[hh][cc][j] = (__bf16)0.f;
     }
-    m2[hh] = (a.sink && hh < nh) ? a.sink[h0 + hh] * kLog2e : -INFINITY;
+    m2[hh] = (!SPLIT && a.sink && hh < nh) ? a.sink[h0 + hh] * kLog2e : -INFINITY;
     l[hh] = 0.f;
 #pragma unroll
     for (int dt = 0; dt < NV; ++dt) o[hh][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -330,7 +348,7 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
     ofv = kbv - pi * a.BS;
     pgv = bi < nblk ? pages[pi] : 0;
   };
-  fill_pages(0);
+  fill_pages(b_lo);
   auto load_k = [&](int page, int off) {
     const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK + g * D + 8 * hq;
 #pragma unroll
@@ -348,9 +366,9 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   int kb_next = __shfl(kbv, 0, 64), pg_next = __shfl(pgv, 0, 64), of_next = __shfl(ofv, 0, 64);
   load_k(pg_next, of_next);
   load_v(pg_next, of_next);
-  for (int bi = 0; bi < nblk; ++bi) {
+  for (int bi = b_lo; bi < b_hi; ++bi) {
     const int kb = kb_next;
-    if (bi + 1 < nblk) {
+    if (bi + 1 < b_hi) {
       if (bi + 1 - pg_base == 64) fill_pages(bi + 1);
       kb_next = __shfl(kbv, bi + 1 - pg_base, 64);
       pg_next = __shfl(pgv, bi + 1 - pg_base, 64);
@@ -370,7 +388,7 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
         for (int i = 0; i < 4; ++i) p[hh][4 * t + i] = sacc[i];
       }
     }
-    if (bi + 1 < nblk) load_k(pg_next, of_next);
+    if (bi + 1 < b_hi) load_k(pg_next, of_next);
     bf16x8 pf[HW];
 #pragma unroll
     for (int hh = 0; hh < HW; ++hh) {
@@ -427,7 +445,7 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
     for (int hh = 0; hh < HW; ++hh)
 #pragma unroll
       for (int dt = 0; dt < NV; ++dt) o[hh][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[hh], vf[dt], o[hh][dt], 0, 0, 0);
-    if (bi + 1 < nblk) load_v(pg_next, of_next);
+    if (bi + 1 < b_hi) load_v(pg_next, of_next);
   }
 #pragma unroll
   for (int hh = 0; hh < HW; ++hh) {
@@ -435,6 +453,23 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
       float lt = l[hh];
       lt += __shfl_xor(lt, 16, 64);
       lt += __shfl_xor(lt, 32, 64);
+      if (SPLIT) {
+        if (hq == 0) {
+          float* ml = a.pml + ((((size_t)item * a.n_parts + blockIdx.z) * H + h0 + hh) * 16 + r) * 2;
+          ml[0] = m2[hh];
+          ml[1] = lt;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int qi = 4 * hq + i;
+          if (qi < ntok) {
+            float* op = a.po + (((size_t)item * a.n_parts + blockIdx.z) * 16 + qi) * H * V + (size_t)(h0 + hh) * V + r;
+#pragma unroll
+            for (int dt = 0; dt < NV; ++dt) op[16 * dt] = o[hh][dt][i];
+          }
+        }
+        continue;
+      }
       if (a.sink) lt += __builtin_amdgcn_exp2f(a.sink[h0 + hh] * kLog2e - m2[hh]);
       const float inv = 1.f / lt;
 #pragma unroll
@@ -452,15 +487,50 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   }
 }
 
-template <int NDC, int NV, int HW>
-static int launch_mask_hw(const MaskArgs& a, int n_items, hipStream_t s) {
+// out[row][h][:] = sum_p o_p 2^(m_p - M) / (sum_p l_p 2^(m_p - M) + 2^(sink - M)) * sigmoid(gate), parts in order
+__global__ void __launch_bounds__(256) masked_attn_merge_kernel(MaskArgs a, int V) {
+  constexpr float kLog2e = 1.4426950408889634f;
+  const int item = blockIdx.x;
+  const int row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2];
+  const int H = a.H, HV = H * V;
+  for (int e = blockIdx.y * 256 + threadIdx.x; e < ntok * HV; e += gridDim.y * 256) {
+    const int q = e / HV, c = e - q * HV, h = c / V;
+    const float sk = a.sink ? a.sink[h] * kLog2e : -INFINITY;
+    float M = sk;
+    for (int p2 = 0; p2 < a.n_parts; ++p2)
+      M = fmaxf(M, a.pml[((((size_t)item * a.n_parts + p2) * H + h) * 16 + q) * 2]);
+    float L = a.sink ? __builtin_amdgcn_exp2f(sk - M) : 0.f, acc = 0.f;
+    for (int p2 = 0; p2 < a.n_parts; ++p2) {
+      const float* ml = a.pml + ((((size_t)item * a.n_parts + p2) * H + h) * 16 + q) * 2;
+      if (ml[0] == -INFINITY) continue;                    // an empty part, or one whose keys this row does not see
+      const float w = __builtin_amdgcn_exp2f(ml[0] - M);
+      L = fmaf(ml[1], w, L);
+      acc = fmaf(a.po[(((size_t)item * a.n_parts + p2) * 16 + q) * HV + c], w, acc);
+    }
+    float f = 1.f / L;
+    if (a.gate) f *= 1.f / (1.f + __expf(-a.gate[(size_t)(row0 + q) * a.gs + h]));
+    a.out[(size_t)(row0 + q) * HV + c] = f2bf(acc * f);
+  }
+}
+
+template <int NDC, int NV, int HW, bool CAP>
+static int launch_mask_cap(const MaskArgs& a, int n_items, hipStream_t s) {
   const int waves_all = (a.H + HW - 1) / HW;               // HW heads per wave, up to eight waves per workgroup
   const int gy = (waves_all + 7) / 8, waves = gy > 1 ? 8 : waves_all;
-  if (a.softcap > 0.f)
-    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, true>), dim3(n_items, gy), dim3(64 * waves), 0, s, a);
-  else
-    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, false>), dim3(n_items, gy), dim3(64 * waves), 0, s, a);
+  if (a.n_parts > 1) {
+    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, CAP, true>), dim3(n_items, gy, a.n_parts), dim3(64 * waves),
+                       0, s, a);
+    hipLaunchKernelGGL(masked_attn_merge_kernel, dim3(n_items, 8), dim3(256), 0, s, a, NV * 16);
+  } else {
+    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, CAP, false>), dim3(n_items, gy), dim3(64 * waves), 0, s, a);
+  }
   return (int)hipGetLastError();
+}
+
+template <int NDC, int NV, int HW>
+static int launch_mask_hw(const MaskArgs& a, int n_items, hipStream_t s) {
+  return a.softcap > 0.f ? launch_mask_cap<NDC, NV, HW, true>(a, n_items, s)
+                         : launch_mask_cap<NDC, NV, HW, false>(a, n_items, s);
 }
 
 // two heads per wave where the heads of a key / value head come in pairs, else one
@@ -521,10 +591,11 @@ K8S_API int k8s_masked_attn_mfma_ok(int H, int G, int D, int V) {
 K8S_API int k8s_masked_attn_mfma(const void* q, const void* kc, const void* vt, const int* block_tables, int maxb,
                                  const int* items, int n_items, const float* sink, const float* gate, int gs, void* out,
                                  int H, int G, int D, int V, int BS, int chunk, int window, int keep_first, float scale,
-                                 float softcap, hipStream_t s) {
+                                 float softcap, hipStream_t s, int part_blocks, int n_parts, float* pml, float* po) {
   if (n_items <= 0) return 0;
   if (!k8s_masked_attn_mfma_ok(H, G, D, V) || BS % 32 || chunk < 0 || window < 0 || keep_first < 0)
     return (int)hipErrorInvalidValue;
+  if (n_parts > 1 && (part_blocks < 1 || !pml || !po)) return (int)hipErrorInvalidValue;
   MaskArgs a;
   a.q = (const uint16_t*)q;
   a.kc = (const uint16_t*)kc;
@@ -545,6 +616,10 @@ K8S_API int k8s_masked_attn_mfma(const void* q, const void* kc, const void* vt, 
   a.keep_first = keep_first;
   a.scale = scale;
   a.softcap = softcap;
+  a.part_blocks = n_parts > 1 ? part_blocks : 1;
+  a.n_parts = n_parts > 1 ? n_parts : 1;
+  a.pml = pml;
+  a.po = po;
   if (D == 64 && V == 64) return launch_mask_mfma<2, 4>(a, n_items, s);
   if (D == 64 && V == 128) return launch_mask_mfma<2, 8>(a, n_items, s);
   if (D == 128 && V == 64) return launch_mask_mfma<4, 4>(a, n_items, s);

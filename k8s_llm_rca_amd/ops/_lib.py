@@ -115,7 +115,7 @@ _SIGS = {
     "k8s_attn_prep": [P, I, P, I, I, I, I, P, P, P, P, P, I, P, I, I, P, P, F, I, F, F, P, P, I, P],
     "k8s_masked_attn_rows": [P, P, P, P, I, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, I, F, F, I, P],
     "k8s_masked_attn_mfma_ok": [I, I, I, I],
-    "k8s_masked_attn_mfma": [P, P, P, P, I, P, I, P, P, I, P, I, I, I, I, I, I, I, I, F, F, P],
+    "k8s_masked_attn_mfma": [P, P, P, P, I, P, I, P, P, I, P, I, I, I, I, I, I, I, I, F, F, P, I, I, P, P],
     "k8s_gated_delta": [P, I, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, P, P, I, P, P, P],
     "k8s_matrix_memory": [P, I, P, F, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P, P, I, P, P, P, P],
     "k8s_head_norm_gate": [P, P, I, P, I, P, I, I, I, F, I, P, P],

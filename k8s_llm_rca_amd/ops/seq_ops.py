@@ -685,11 +685,27 @@ def masked_attention(q: torch.Tensor, H: int, G: int, D: int, V: int, kc: torch.
         if vt is not None and masked_mfma_ok(H, G, D, V, q.dtype, q.device):
             assert vt.is_contiguous() and vt.shape[1:] == (G * V, BS) and BS % 32 == 0
             items = seg.tile_items(WINDOW_TILE)
+            n_items = items.shape[0]
+            # steps of few rows (decoding): a tile's key blocks are split over workgroups as well -- parts of
+            # MASK_PART_BLOCKS blocks of the tile's own block list (at most MASK_MAX_PARTS parts), then a merge
+            n_parts, pb, pml, po = 1, MASK_PART_BLOCKS, None, None
+            if n_items <= WINDOW_SPLIT_ITEMS:
+                kmax = max(p + b - a for p, a, b in zip(seg.pos0_host, seg.row0_host[:-1], seg.row0_host[1:]))
+                nblk = -(-kmax // 32) + 1                  # an upper bound of any tile's blocks
+                if window > 0:     # a tile's span: the window, its 16 tokens, a block's alignment; + the kept blocks
+                    nblk = min(nblk, (int(window) + 45) // 32 + 1 + -(-int(keep_first) // 32))
+                if chunk > 0:
+                    nblk = min(nblk, (int(chunk) + 45) // 32 + 1)
+                pb = max(MASK_PART_BLOCKS, -(-nblk // MASK_MAX_PARTS))
+                n_parts = -(-nblk // pb)
+                if n_parts > 1:
+                    pml = scratch(n_items * n_parts * H * 32, torch.float32, q.device)
+                    po = scratch(n_items * n_parts * 16 * H * V, torch.float32, q.device)
             check(lib().k8s_masked_attn_mfma(ptr(q), ptr(kc), ptr(vt), ptr(seg.block_tables),
-                                             seg.block_tables.shape[1], ptr(items), items.shape[0], ptr(sink),
+                                             seg.block_tables.shape[1], ptr(items), n_items, ptr(sink),
                                              ptr(gate), gs, ptr(out), H, G, D, V, BS, int(chunk), int(window),
-                                             int(keep_first), float(scale), float(softcap), stream_ptr(q)),
-                  "masked_attn_mfma")
+                                             int(keep_first), float(scale), float(softcap), stream_ptr(q), pb, n_parts,
+                                             ptr(pml), ptr(po)), "masked_attn_mfma")
             return out
         check(lib().k8s_masked_attn_rows(ptr(q), ptr(kc), ptr(vc), ptr(seg.block_tables), seg.block_tables.shape[1],
                                          ptr(seg.row_seg), ptr(seg.seg_row0), ptr(seg.seg_pos0), ptr(sink), ptr(gate),
@@ -728,6 +744,10 @@ def masked_attention(q: torch.Tensor, H: int, G: int, D: int, V: int, kc: torch.
             o = o * torch.sigmoid(gate[a:e, :H])[:, :, None]
         out[a:e] = o.reshape(n, H * V).to(q.dtype)
     return out
+
+
+MASK_PART_BLOCKS = 4    # 32-key blocks per part when a step of few rows is split over the keys too
+MASK_MAX_PARTS = 32
 
 
 def masked_mfma_ok(H: int, G: int, D: int, V: int, dtype, device) -> bool:

@@ -382,10 +382,14 @@ MFMA_BACKEND = [pytest.param(("cuda", torch.bfloat16), id="gpu-bf16", marks=GPU)
 @pytest.mark.parametrize("backend", MFMA_BACKEND)
 @pytest.mark.parametrize("H,G,D,V", [(4, 2, 64, 64), (3, 1, 128, 64), (18, 2, 64, 128), (2, 2, 128, 128), (1, 1, 64, 64)])
 @pytest.mark.parametrize("mask", range(len(MASKS)))
-def test_masked_attention_on_the_matrix_cores(backend, H, G, D, V, mask):
+@pytest.mark.parametrize("split", [True, False])
+def test_masked_attention_on_the_matrix_cores(backend, H, G, D, V, mask, split, monkeypatch):
     """The sizes the matrix-core kernel takes: tiles of 16 tokens, portions that start inside a tile's
-    span, a chunk border inside a tile, decoding token by token."""
+    span, a chunk border inside a tile, decoding token by token; with and without the split of a tile's key
+    blocks over workgroups that steps of few rows get."""
     dev, dt = backend
+    if not split:
+        monkeypatch.setattr(S, "WINDOW_SPLIT_ITEMS", 0)
     mk = MASKS[mask]
     n, BS, scale = 150, 32, 0.25
     q, k, v, kc, vc, bt, vt = attention_case(dev, dt, H, G, D, V, n, BS, seed=mask + H, with_twin=True)
@@ -410,6 +414,35 @@ def test_masked_attention_on_the_matrix_cores(backend, H, G, D, V, mask):
     got = S.masked_attention(torch.cat([qd[n - 5:], qd[100:]]).contiguous(), H, G, D, V, kc, vc, sg, scale,
                              gate=None if gd is None else torch.cat([gd[n - 5:], gd[100:]])[:, 1:], vt=vt, **kw)
     close(got, torch.cat([want[n - 5:], want[100:]]).reshape(n - 95, -1), dt)
+
+
+@pytest.mark.parametrize("backend", MFMA_BACKEND)
+@pytest.mark.parametrize("mk", [dict(), dict(window=2100, keep_first=70), dict(chunk=2112, softcap=3.0)])
+def test_masked_attention_many_blocks(backend, mk):
+    """More than 64 key blocks per tile (the block table is refilled), as a whole prompt and for the last
+    tokens alone (many parts).  The expected values are a dense softmax in float64."""
+    dev, dt = backend
+    H, G, D, V, n, BS, scale = 2, 1, 64, 64, 2200, 64, 0.2
+    q, k, v, kc, vc, bt, vt = attention_case(dev, dt, H, G, D, V, n, BS, seed=7, with_twin=True)
+    sc = torch.einsum("ihd,jd->hij", q, k[:, 0]) * scale
+    if mk.get("softcap"):
+        sc = mk["softcap"] * torch.tanh(sc / mk["softcap"])
+    i, j = torch.arange(n)[:, None], torch.arange(n)[None, :]
+    vis = j <= i
+    if mk.get("chunk"):
+        vis &= (i // mk["chunk"]) == (j // mk["chunk"])
+    if mk.get("window"):
+        vis &= ((i - j) < mk["window"]) | (j < mk["keep_first"])
+    want = torch.einsum("hij,jv->ihv", torch.softmax(sc.masked_fill(~vis, float("-inf")), -1), v[:, 0]).reshape(n, -1)
+    qd = q.reshape(n, -1).to(dev).to(dt)
+    kw = dict(softcap=mk.get("softcap", 0.0), chunk=mk.get("chunk", 0), window=mk.get("window", 0),
+              keep_first=mk.get("keep_first", 0))
+    got = S.masked_attention(qd, H, G, D, V, kc, vc, seg_meta([n], [0], [0], dev, bt), scale, vt=vt, **kw)
+    close(got, want, dt)
+    for a in (n - 1, n - 3, n - 40):
+        got = S.masked_attention(qd[a:].contiguous(), H, G, D, V, kc, vc, seg_meta([n - a], [a], [0], dev, bt), scale,
+                                 vt=vt, **kw)
+        close(got, want[a:], dt)
 
 
 @pytest.mark.parametrize("backend", MFMA_BACKEND)
