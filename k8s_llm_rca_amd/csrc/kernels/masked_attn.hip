@@ -47,12 +47,11 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const float* __restrict_
                                                         TA* __restrict__ q_out, int norm, const float* __restrict__ q_w,
                                                         const float* __restrict__ k_w, float eps, int rot, float base,
                                                         float lam, const float* __restrict__ v_other,
-                                                        float* __restrict__ v_keep) {
-  extern __shared__ float sm[];   // [rot]: cos | sin;  [4][D]: one head per wave
+                                                        float* __restrict__ v_keep, int upr) {
+  extern __shared__ float sm[];   // [rot]: cos | sin;  [upr][D]: the heads of one round
   const int r = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int half = rot >> 1;
   float* cs = sm;
-  float* buf = sm + rot + wv * D;
   if (rot) {
     const double lb = log((double)base), p = (double)positions[r];
     for (int i = tid; i < half; i += 256) {
@@ -64,12 +63,17 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const float* __restrict_
   const int sl = slots[r];
   const int NQ = H * D, NK = G * D, NV = G * V, units = H + G;
   const float* row = qkv + (size_t)r * qs;
-  for (int u0 = 0; u0 < units; u0 += 4) {      // every wave takes the same number of turns (barriers inside)
-    const int u = u0 + wv;
-    if (u < units)
+  // rounds of upr heads (all of the row's q and k heads where LDS holds them: one barrier pair per row):
+  // the round's heads are loaded, then every wave works on its own
+  for (int u0 = 0; u0 < units; u0 += upr) {
+    const int u1 = min(units, u0 + upr);
+    for (int u = u0 + wv; u < u1; u += 4) {
+      float* buf = sm + rot + (u - u0) * D;
       for (int d = lane; d < D; d += 64) buf[d] = row[u * D + d] + (bias ? bias[u * D + d] : 0.f);
+    }
     __syncthreads();
-    if (u < units) {
+    for (int u = u0 + wv; u < u1; u += 4) {
+      const float* buf = sm + rot + (u - u0) * D;
       float val[kPrepPer];
       float ss = 0.f;
 #pragma unroll
@@ -103,7 +107,7 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const float* __restrict_
         }
       }
     }
-    __syncthreads();
+    if (u1 < units) __syncthreads();
   }
   const int page = sl >= 0 ? sl / BS : 0, off = sl >= 0 ? sl - page * BS : 0;
   for (int c = tid; c < NV; c += 256) {
@@ -550,15 +554,17 @@ K8S_API int k8s_attn_prep(const float* qkv, int qs, const float* bias, int H, in
   if (T <= 0) return 0;
   if (H < 1 || G < 1 || D < 1 || D > 64 * kPrepPer || V < 1 || rot < 0 || rot > D || (rot & 1) || BS < 1)
     return (int)hipErrorInvalidValue;
-  const size_t lds = (size_t)(rot + 4 * D) * sizeof(float);
+  const int units = H + G;
+  const int upr = (size_t)(rot + units * D) * sizeof(float) <= 64 * 1024 ? units : 4;    // heads per round
+  const size_t lds = (size_t)(rot + upr * D) * sizeof(float);
   if (dt == 0)
     hipLaunchKernelGGL((attn_prep_kernel<uint16_t>), dim3(T), dim3(256), lds, s, qkv, qs, bias, H, G, D, V, positions,
                        slots, (uint16_t*)kc, (uint16_t*)vc, (uint16_t*)vt, BS, (uint16_t*)q_out, norm, q_w, k_w, eps, rot,
-                       base, lam, v_other, v_keep);
+                       base, lam, v_other, v_keep, upr);
   else
     hipLaunchKernelGGL((attn_prep_kernel<float>), dim3(T), dim3(256), lds, s, qkv, qs, bias, H, G, D, V, positions, slots,
                        (float*)kc, (float*)vc, (float*)vt, BS, (float*)q_out, norm, q_w, k_w, eps, rot, base, lam,
-                       v_other, v_keep);
+                       v_other, v_keep, upr);
   return (int)hipGetLastError();
 }
 

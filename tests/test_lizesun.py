@@ -259,7 +259,7 @@ def slots_of(order, BS, a, e, dev):
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("H,G,D,V,rot,norm,wts", [(4, 2, 8, 12, 4, True, False), (3, 3, 6, 5, 6, True, True),
                                                   (2, 1, 16, 8, 0, True, True), (5, 1, 70, 3, 32, False, False),
-                                                  (1, 1, 4, 130, 2, True, False)])
+                                                  (1, 1, 4, 130, 2, True, False), (40, 8, 400, 3, 64, True, True)])
 def test_attention_preparation(backend, H, G, D, V, rot, norm, wts):
     """Bias, rotation far from position 0, unit norm with and without a weight, value mixing, paged write."""
     dev, dt = backend
