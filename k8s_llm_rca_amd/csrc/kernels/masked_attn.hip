@@ -141,7 +141,7 @@ __device__ __forceinline__ KeyRuns key_runs(int pos, int chunk, int window, int 
 }
 
 constexpr int kMaskTile = 64;   // keys per tile: one per lane
-constexpr int kMaskOut = 16;    // outputs per thread: H * V <= 256 * kMaskOut
+constexpr int kMaskOut = 32;    // outputs per thread: H * V <= 256 * kMaskOut
 
 template <typename TA>
 __device__ __forceinline__ float mask_score(const float* q, const TA* __restrict__ kc, const int* __restrict__ bt, int BS,

@@ -326,7 +326,7 @@ def visible(chunk=0, window=0, keep_first=0, **_):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("H,G,D,V", [(4, 2, 8, 12), (3, 3, 5, 3), (6, 1, 32, 16), (1, 1, 64, 70)])
+@pytest.mark.parametrize("H,G,D,V", [(4, 2, 8, 12), (3, 3, 5, 3), (6, 1, 32, 16), (1, 1, 64, 70), (24, 4, 16, 200)])
 @pytest.mark.parametrize("mask", range(len(MASKS)))
 def test_masked_attention_paged(backend, H, G, D, V, mask):
     dev, dt = backend
