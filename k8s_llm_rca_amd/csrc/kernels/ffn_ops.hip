@@ -78,18 +78,22 @@ __global__ void __launch_bounds__(256) glu_clamp_kernel(const TA* __restrict__ g
 // Router: one wave per token.  logits = Wr h in fp32; scores = sigmoid(logits)
 // (mode 0) or softmax (mode 1); the K largest (ties: lowest index), optionally
 // renormalised to sum 1 (divided by their sum + renorm_eps).  With `bias` [E] the
-// choice is made on score + bias while the weights stay the plain scores.
+// choice is made on score + bias while the weights stay the plain scores.  The weights are multiplied by
+// out_scale at the end.  wr may hold X more rows behind the E experts' (Et = E + X): their logits are not
+// routed but written as they are to extra[t][X] (per-token gates that read the same hidden row).
 template <typename TA, typename TW>
 __global__ void __launch_bounds__(256) router_kernel(const TA* __restrict__ h, const TW* __restrict__ wr, int T, int W,
-                                                     int E, int K, int mode, int renorm, float* __restrict__ w_out,
+                                                     int Et, int K, int mode, int renorm, float* __restrict__ w_out,
                                                      int* __restrict__ id_out, const float* __restrict__ bias,
-                                                     float renorm_eps) {
+                                                     float renorm_eps, int X, float* __restrict__ extra,
+                                                     float out_scale) {
   extern __shared__ float sm[];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int t = blockIdx.x * 4 + wv;
   if (t >= T) return;
-  float* sc = sm + wv * 2 * E;
-  float* ch = sc + E;   // choice scores
+  float* sc = sm + wv * 2 * Et;
+  float* ch = sc + Et;   // choice scores
+  const int E = Et;      // rows whose logits are formed below; the routed ones are E - X
   if ((W & 7) == 0) {
     // 8 columns per lane and step, 16 experts at a time: the hidden row is read once per group
     for (int e0 = 0; e0 < E; e0 += 16) {
@@ -125,6 +129,8 @@ __global__ void __launch_bounds__(256) router_kernel(const TA* __restrict__ h, c
   }
   __builtin_amdgcn_wave_barrier();
   if (lane == 0) {
+    const int E = Et - X;
+    for (int x = 0; x < X; ++x) extra[(size_t)t * X + x] = sc[E + x];
     if (mode == 0) {
       for (int e = 0; e < E; ++e) sc[e] = 1.f / (1.f + expf(-sc[e]));
     } else {
@@ -150,6 +156,8 @@ __global__ void __launch_bounds__(256) router_kernel(const TA* __restrict__ h, c
     }
     if (renorm)
       for (int k = 0; k < K; ++k) w_out[t * K + k] /= (tot + renorm_eps);
+    if (out_scale != 1.f)
+      for (int k = 0; k < K; ++k) w_out[t * K + k] *= out_scale;
   }
 }
 
@@ -269,12 +277,13 @@ K8S_API int k8s_glu_clamp(const void* gu, void* out, int rows, int F, float alph
 }
 
 K8S_API int k8s_router(const void* h, const void* wr, int T, int W, int E, int K, int mode, int renorm, float* w_out,
-                       int* id_out, int dt, hipStream_t s, const float* bias, float renorm_eps) {
+                       int* id_out, int dt, hipStream_t s, const float* bias, float renorm_eps, int X, float* extra,
+                       float out_scale) {
   if (T <= 0) return 0;
-  if (K > E || E > 2048) return (int)hipErrorInvalidValue;
-  K8S_DT(dt, hipLaunchKernelGGL((router_kernel<TA, TW>), dim3((T + 3) / 4), dim3(256), 8 * E * sizeof(float), s,
-                                 (const TA*)h, (const TW*)wr, T, W, E, K, mode, renorm, w_out, id_out, bias,
-                                 renorm_eps));
+  if (K > E || E + X > 2048 || X < 0 || (X > 0 && !extra)) return (int)hipErrorInvalidValue;
+  K8S_DT(dt, hipLaunchKernelGGL((router_kernel<TA, TW>), dim3((T + 3) / 4), dim3(256), 8 * (E + X) * sizeof(float), s,
+                                 (const TA*)h, (const TW*)wr, T, W, E + X, K, mode, renorm, w_out, id_out, bias,
+                                 renorm_eps, X, extra, out_scale));
   return (int)hipGetLastError();
 }
 

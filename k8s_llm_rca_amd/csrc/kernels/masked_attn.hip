@@ -1,17 +1,26 @@
 // Softmax attention over a paged key / value cache under a position mask, behind a pass that prepares
 // q and k.
 //
-// attn_prep:  rows of the joint projection (fp32: q [H][D] | k [G][D] | v [G][V], row stride qs)
+// attn_prep:  rows of the joint projection (fp32: q [H][D] | k [G][D] | v [NV], row stride qs)
 //   + bias;  q, k rotated on their first `rot` entries per head (entry i with i + rot / 2, angle
-//   pos * base^(-2 i / rot), formed in double);  q, k divided by the head's root mean square (eps inside the
-//   root) and multiplied by a weight [D] where given;  v optionally kept as projected (v_keep) and mixed
-//   with another layer's values of the same token, (1 - lam) v + lam v_other;  k and v written to their pages
-//   (and v to the transposed twin), q written as activations.
+//   pos * base^(-2 i / rot), formed in double);  norm 1: q, k divided by the head's root mean square (eps inside
+//   the root) behind the rotation and multiplied by a weight [D] where given;  norm 2: q and k each divided by
+//   the root mean square of the WHOLE projection (all heads at once) and multiplied by a weight of that size,
+//   in front of the rotation;  q multiplied by the position's temperature 1 + tq_coef ln(floor((pos + 1) /
+//   tq_every) + 1) (tq_every > 0);  v optionally kept as projected (v_keep) and mixed with another layer's
+//   values of the same token, (1 - lam) v + lam v_other;  k and v written to their pages (and v to the
+//   transposed twin), q written as activations.  The values start at column v_col of the row: behind the
+//   keys, or AT the keys (the values are the keys as projected).  G = 0: a layer that reads another layer's
+//   pages prepares its queries only.  H and G count heads of D entries: a layer with several score maps per
+//   head passes maps * heads.
 //
 // masked attention:  position i sees j <= i with  (chunk > 0:  i / chunk == j / chunk)  and
 //   (window > 0:  i - j < window  or  j < keep_first).  s = scale q.k, then softcap tanh(s / softcap) for
 //   softcap > 0.  A sink adds exp(sink_h) to head h's denominator.  Head h's output may be multiplied by
-//   sigmoid(gate[t][h]).  Query head h reads key / value head h / (H / G).
+//   sigmoid(gate[t][h]).  Query head h reads key / value head h / (H / G).  With M > 1 score maps per head, q
+//   holds H M heads laid out [h][m] and the key pages G M heads [g][m]: map m of head h scores against key
+//   head (h / (H / G)) M + m and applies its weights to value head h / (H / G); the output is [T][H][M][V],
+//   each map's result by itself (fp32 where the caller joins the maps).
 //   The visible keys of a row are two runs, [a0, a1) (kept first tokens) and [lo, pos]; both kernels walk
 //   them as one virtual range whose tile borders depend on the row's position only, so a row's result
 //   does not depend on how the prompt was cut or on what else is in the step.
@@ -40,15 +49,17 @@ constexpr int kPrepPer = 8;    // entries of a head per lane: D <= 512
 
 template <typename TA>
 __global__ void __launch_bounds__(256) attn_prep_kernel(const float* __restrict__ qkv, int qs,
-                                                        const float* __restrict__ bias, int H, int G, int D, int V,
+                                                        const float* __restrict__ bias, int H, int G, int D, int NV,
                                                         const int* __restrict__ positions,
                                                         const int* __restrict__ slots, TA* __restrict__ kc,
                                                         TA* __restrict__ vc, TA* __restrict__ vt, int BS,
                                                         TA* __restrict__ q_out, int norm, const float* __restrict__ q_w,
                                                         const float* __restrict__ k_w, float eps, int rot, float base,
                                                         float lam, const float* __restrict__ v_other,
-                                                        float* __restrict__ v_keep, int upr) {
+                                                        float* __restrict__ v_keep, int upr, int v_col, float tq_coef,
+                                                        int tq_every) {
   extern __shared__ float sm[];   // [rot]: cos | sin;  [upr][D]: the heads of one round
+  __shared__ float red[16];
   const int r = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int half = rot >> 1;
   float* cs = sm;
@@ -61,15 +72,35 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const float* __restrict_
     }
   }
   const int sl = slots[r];
-  const int NQ = H * D, NK = G * D, NV = G * V, units = H + G;
+  const int NQ = H * D, NK = G * D, units = H + G;
   const float* row = qkv + (size_t)r * qs;
+  const float tq = tq_every > 0 ? 1.f + tq_coef * logf((float)((positions[r] + 1) / tq_every) + 1.f) : 1.f;
+  // norm 2: 1 / rms of the whole q and of the whole k projection
+  float rq = 1.f, rk = 1.f;
+  if (norm == 2) {
+    float sq = 0.f, sk = 0.f;
+    for (int i = tid; i < NQ; i += 256) {
+      const float v = row[i] + (bias ? bias[i] : 0.f);
+      sq = fmaf(v, v, sq);
+    }
+    for (int i = tid; i < NK; i += 256) {
+      const float v = row[NQ + i] + (bias ? bias[NQ + i] : 0.f);
+      sk = fmaf(v, v, sk);
+    }
+    rq = 1.f / sqrtf(block_sum(sq, red) / (float)NQ + eps);
+    if (NK) rk = 1.f / sqrtf(block_sum(sk, red) / (float)NK + eps);
+  }
   // rounds of upr heads (all of the row's q and k heads where LDS holds them: one barrier pair per row):
   // the round's heads are loaded, then every wave works on its own
   for (int u0 = 0; u0 < units; u0 += upr) {
     const int u1 = min(units, u0 + upr);
     for (int u = u0 + wv; u < u1; u += 4) {
       float* buf = sm + rot + (u - u0) * D;
-      for (int d = lane; d < D; d += 64) buf[d] = row[u * D + d] + (bias ? bias[u * D + d] : 0.f);
+      for (int d = lane; d < D; d += 64) {
+        float v = row[u * D + d] + (bias ? bias[u * D + d] : 0.f);
+        if (norm == 2) v *= u < H ? rq * (q_w ? q_w[u * D + d] : 1.f) : rk * (k_w ? k_w[(u - H) * D + d] : 1.f);
+        buf[d] = v;
+      }
     }
     __syncthreads();
     for (int u = u0 + wv; u < u1; u += 4) {
@@ -93,8 +124,9 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const float* __restrict_
         ss = fmaf(xv, xv, ss);
       }
       float rn = 1.f;
-      if (norm) rn = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
-      const float* wgt = u < H ? q_w : k_w;
+      if (norm == 1) rn = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+      const float* wgt = norm == 1 ? (u < H ? q_w : k_w) : nullptr;
+      if (u < H) rn *= tq;
 #pragma unroll
       for (int i = 0; i < kPrepPer; ++i) {
         const int d = lane + 64 * i;
@@ -111,7 +143,7 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const float* __restrict_
   }
   const int page = sl >= 0 ? sl / BS : 0, off = sl >= 0 ? sl - page * BS : 0;
   for (int c = tid; c < NV; c += 256) {
-    float v = row[NQ + NK + c] + (bias ? bias[NQ + NK + c] : 0.f);
+    float v = row[v_col + c] + (bias ? bias[v_col + c] : 0.f);
     if (v_keep) v_keep[(size_t)r * NV + c] = v;
     if (v_other) v = (1.f - lam) * v + lam * v_other[(size_t)r * NV + c];
     if (sl >= 0) {
@@ -156,7 +188,7 @@ __device__ __forceinline__ float mask_score(const float* q, const TA* __restrict
 // One workgroup per row, two passes over the row's visible keys in tiles of 64:
 //   1. per head the maximum (the sink included) and the denominator, online (a wave per head);
 //   2. scores again -> weights in LDS -> times the values (a thread per output column).
-template <typename TA>
+template <typename TA, typename TO>
 __global__ void __launch_bounds__(256) masked_attn_rows_kernel(const TA* __restrict__ q, const TA* __restrict__ kc,
                                                                const TA* __restrict__ vc,
                                                                const int* __restrict__ block_tables, int maxb,
@@ -165,9 +197,10 @@ __global__ void __launch_bounds__(256) masked_attn_rows_kernel(const TA* __restr
                                                                const int* __restrict__ seg_pos0,
                                                                const float* __restrict__ sink,
                                                                const float* __restrict__ gate, int gs,
-                                                               TA* __restrict__ out, int H, int G, int D, int V, int BS,
+                                                               TO* __restrict__ out, int H, int G, int D, int V, int BS,
                                                                int chunk, int window, int keep_first, float scale,
-                                                               float softcap) {
+                                                               float softcap, int M) {
+  // H counts the query heads of D entries (heads x maps); hpg of them share a key / value head group
   extern __shared__ float sm[];
   float* qf = sm;                      // [H][D]
   float* p = qf + H * D;               // [H][64]
@@ -177,11 +210,11 @@ __global__ void __launch_bounds__(256) masked_attn_rows_kernel(const TA* __restr
   const int sg = row_seg[r], pos = seg_pos0[sg] + r - seg_row0[sg];
   const KeyRuns kr = key_runs(pos, chunk, window, keep_first);
   const int* bt = block_tables + (size_t)sg * maxb;
-  const int NK = G * D, NV = G * V, hpg = H / G;
+  const int NK = G * M * D, NV = G * V, hpg = H / (G * M);
   for (int i = tid; i < H * D; i += 256) qf[i] = lda(q, (size_t)r * H * D + i);
   __syncthreads();
   for (int h = wv; h < H; h += 4) {
-    const int g = h / hpg;
+    const int g = (h / M / hpg) * M + h % M;
     float m = sink ? sink[h] : -INFINITY, l = sink ? 1.f : 0.f;
     for (int x0 = 0; x0 < kr.total; x0 += kMaskTile) {
       const int x = x0 + lane;
@@ -204,7 +237,8 @@ __global__ void __launch_bounds__(256) masked_attn_rows_kernel(const TA* __restr
     for (int h = wv; h < H; h += 4) {
       const int x = x0 + lane;
       const bool ok = x < kr.total;
-      const float s = ok ? mask_score(qf + h * D, kc, bt, BS, NK, D, h / hpg, kr.key(x), scale, softcap) : 0.f;
+      const float s =
+          ok ? mask_score(qf + h * D, kc, bt, BS, NK, D, (h / M / hpg) * M + h % M, kr.key(x), scale, softcap) : 0.f;
       p[h * kMaskTile + lane] = ok ? expf(s - mh[h]) / lh[h] : 0.f;
     }
     __syncthreads();
@@ -213,7 +247,7 @@ __global__ void __launch_bounds__(256) masked_attn_rows_kernel(const TA* __restr
     for (int i = 0; i < kMaskOut; ++i) {
       const int o = tid + i * 256;
       if (o < H * V) {
-        const int h = o / V, v = o - h * V, g = h / hpg;
+        const int h = o / V, v = o - h * V, g = h / M / hpg;
         float a = acc[i];
         for (int jj = 0; jj < nk; ++jj) {
           const int j = kr.key(x0 + jj);
@@ -230,7 +264,7 @@ __global__ void __launch_bounds__(256) masked_attn_rows_kernel(const TA* __restr
     if (o < H * V) {
       float a = acc[i];
       if (gate) a *= 1.f / (1.f + expf(-gate[(size_t)r * gs + o / V]));
-      sta(out, (size_t)r * H * V + o, a);
+      sta(out, (size_t)r * H * V + o, a);   // (gates count heads x maps like H)
     }
   }
 }
@@ -258,7 +292,8 @@ struct MaskArgs {
   const float* gate;      // [T] rows of stride gs, column h, or null
   int gs;
   uint16_t* out;          // [T][H * V]
-  int H, G, BS, chunk, window, keep_first;
+  float* out32;           // the same in fp32 instead, where the caller joins score maps
+  int H, G, M, BS, chunk, window, keep_first;   // H: query heads of D entries (heads x M maps)
   float scale, softcap;
   // steps of few rows: a tile's key blocks are split over grid.z workgroups, part_blocks blocks each
   int part_blocks, n_parts;
@@ -282,7 +317,7 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   const int item = a.n_items - 1 - blockIdx.x;
   const int sg = a.items[item * 4], row0 = a.items[item * 4 + 1], ntok = a.items[item * 4 + 2],
             pos0 = a.items[item * 4 + 3];
-  const int H = a.H, hpg = H / a.G, NK = a.G * D, NVt = a.G * V;
+  const int H = a.H, hpg = H / (a.G * a.M), NK = a.G * a.M * D, NVt = a.G * V;
   const int h0 = (blockIdx.y * 8 + wv) * HW, nh = min(HW, H - h0);
   if (nh <= 0) return;                                     // the whole wave; nothing below synchronises waves
   const int posq = pos0 + r, pos_last = pos0 + ntok - 1;
@@ -336,7 +371,8 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   // loads and value loads are dependent memory accesses, so they are issued a block ahead into the SAME
   // registers: the next keys as soon as this block's scores are formed, the next values as soon as this
   // block's value products are issued; the softmax and the products run meanwhile.
-  const int g = h0 / hpg;
+  // (with score maps, HW = 1: map m of a head reads key head m of its group and the group's one value head)
+  const int gv = h0 / a.M / hpg, g = gv * a.M + h0 % a.M;
   bf16x8 kf[2][NDC];
   bf16x8 vf[NV];
   auto block_at = [&](int bi) { return bi < nblkA ? a_beg + 32 * bi : lo_al + 32 * (bi - nblkA); };
@@ -363,7 +399,7 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
     }
   };
   auto load_v = [&](int page, int off) {
-    const uint16_t* vp = a.vt + ((size_t)page * NVt + (size_t)g * V) * a.BS + off + 8 * hq;
+    const uint16_t* vp = a.vt + ((size_t)page * NVt + (size_t)gv * V) * a.BS + off + 8 * hq;
 #pragma unroll
     for (int dt = 0; dt < NV; ++dt) vf[dt] = mld16(vp + (size_t)(16 * dt + r) * a.BS);
   };
@@ -482,9 +518,14 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
         float f = __shfl(inv, qi, 64);
         if (qi < ntok) {
           if (a.gate) f *= 1.f / (1.f + __expf(-a.gate[(size_t)(row0 + qi) * a.gs + h0 + hh]));
-          uint16_t* op = a.out + (size_t)(row0 + qi) * H * V + (size_t)(h0 + hh) * V + r;
+          const size_t oo = (size_t)(row0 + qi) * H * V + (size_t)(h0 + hh) * V + r;
+          if (a.out32) {
 #pragma unroll
-          for (int dt = 0; dt < NV; ++dt) op[16 * dt] = f2bf(o[hh][dt][i] * f);
+            for (int dt = 0; dt < NV; ++dt) a.out32[oo + 16 * dt] = o[hh][dt][i] * f;
+          } else {
+#pragma unroll
+            for (int dt = 0; dt < NV; ++dt) a.out[oo + 16 * dt] = f2bf(o[hh][dt][i] * f);
+          }
         }
       }
     }
@@ -513,7 +554,10 @@ __global__ void __launch_bounds__(256) masked_attn_merge_kernel(MaskArgs a, int 
     }
     float f = 1.f / L;
     if (a.gate) f *= 1.f / (1.f + __expf(-a.gate[(size_t)(row0 + q) * a.gs + h]));
-    a.out[(size_t)(row0 + q) * HV + c] = f2bf(acc * f);
+    if (a.out32)
+      a.out32[(size_t)(row0 + q) * HV + c] = acc * f;
+    else
+      a.out[(size_t)(row0 + q) * HV + c] = f2bf(acc * f);
   }
 }
 
@@ -540,31 +584,34 @@ static int launch_mask_hw(const MaskArgs& a, int n_items, hipStream_t s) {
 // two heads per wave where the heads of a key / value head come in pairs, else one
 template <int NDC, int NV>
 static int launch_mask_mfma(const MaskArgs& a, int n_items, hipStream_t s) {
-  return (a.H / a.G) % 2 == 0 ? launch_mask_hw<NDC, NV, 2>(a, n_items, s) : launch_mask_hw<NDC, NV, 1>(a, n_items, s);
+  return a.M == 1 && (a.H / a.G) % 2 == 0 ? launch_mask_hw<NDC, NV, 2>(a, n_items, s)
+                                          : launch_mask_hw<NDC, NV, 1>(a, n_items, s);
 }
 
 }  // namespace k8s
 
 using namespace k8s;
 
-K8S_API int k8s_attn_prep(const float* qkv, int qs, const float* bias, int H, int G, int D, int V, const int* positions,
+K8S_API int k8s_attn_prep(const float* qkv, int qs, const float* bias, int H, int G, int D, int NV, const int* positions,
                           const int* slots, void* kc, void* vc, void* vt, int BS, void* q_out, int dt, int norm,
                           const float* q_w, const float* k_w, float eps, int rot, float base, float lam,
-                          const float* v_other, float* v_keep, int T, hipStream_t s) {
+                          const float* v_other, float* v_keep, int T, hipStream_t s, int v_col, float tq_coef,
+                          int tq_every) {
   if (T <= 0) return 0;
-  if (H < 1 || G < 1 || D < 1 || D > 64 * kPrepPer || V < 1 || rot < 0 || rot > D || (rot & 1) || BS < 1)
+  if (H < 1 || G < 0 || D < 1 || D > 64 * kPrepPer || NV < 0 || rot < 0 || rot > D || (rot & 1) || BS < 1 ||
+      norm < 0 || norm > 2 || v_col < 0 || tq_every < 0 || ((G > 0 || NV > 0) && (!kc || !vc)))
     return (int)hipErrorInvalidValue;
   const int units = H + G;
   const int upr = (size_t)(rot + units * D) * sizeof(float) <= 64 * 1024 ? units : 4;    // heads per round
   const size_t lds = (size_t)(rot + upr * D) * sizeof(float);
   if (dt == 0)
-    hipLaunchKernelGGL((attn_prep_kernel<uint16_t>), dim3(T), dim3(256), lds, s, qkv, qs, bias, H, G, D, V, positions,
+    hipLaunchKernelGGL((attn_prep_kernel<uint16_t>), dim3(T), dim3(256), lds, s, qkv, qs, bias, H, G, D, NV, positions,
                        slots, (uint16_t*)kc, (uint16_t*)vc, (uint16_t*)vt, BS, (uint16_t*)q_out, norm, q_w, k_w, eps, rot,
-                       base, lam, v_other, v_keep, upr);
+                       base, lam, v_other, v_keep, upr, v_col, tq_coef, tq_every);
   else
-    hipLaunchKernelGGL((attn_prep_kernel<float>), dim3(T), dim3(256), lds, s, qkv, qs, bias, H, G, D, V, positions, slots,
+    hipLaunchKernelGGL((attn_prep_kernel<float>), dim3(T), dim3(256), lds, s, qkv, qs, bias, H, G, D, NV, positions, slots,
                        (float*)kc, (float*)vc, (float*)vt, BS, (float*)q_out, norm, q_w, k_w, eps, rot, base, lam,
-                       v_other, v_keep, upr);
+                       v_other, v_keep, upr, v_col, tq_coef, tq_every);
   return (int)hipGetLastError();
 }
 
@@ -572,20 +619,26 @@ K8S_API int k8s_masked_attn_rows(const void* q, const void* kc, const void* vc, 
                                  const int* row_seg, const int* seg_row0, const int* seg_pos0, const float* sink,
                                  const float* gate, int gs, void* out, int T, int H, int G, int D, int V, int BS,
                                  int chunk, int window, int keep_first, float scale, float softcap, int dt,
-                                 hipStream_t s) {
+                                 hipStream_t s, int maps, int out_f32) {
   if (T <= 0) return 0;
-  const size_t lds = (size_t)(H * D + H * kMaskTile + 2 * H) * sizeof(float);
-  if (H < 1 || G < 1 || H % G || H * V > 256 * kMaskOut || chunk < 0 || window < 0 || keep_first < 0 ||
+  if (maps < 1) return (int)hipErrorInvalidValue;
+  const int HQ = H * maps;
+  const size_t lds = (size_t)(HQ * D + HQ * kMaskTile + 2 * HQ) * sizeof(float);
+  if (H < 1 || G < 1 || H % G || HQ * V > 256 * kMaskOut || chunk < 0 || window < 0 || keep_first < 0 ||
       lds > 64 * 1024)
     return (int)hipErrorInvalidValue;
-  if (dt == 0)
-    hipLaunchKernelGGL((masked_attn_rows_kernel<uint16_t>), dim3(T), dim3(256), lds, s, (const uint16_t*)q,
-                       (const uint16_t*)kc, (const uint16_t*)vc, block_tables, maxb, row_seg, seg_row0, seg_pos0, sink,
-                       gate, gs, (uint16_t*)out, H, G, D, V, BS, chunk, window, keep_first, scale, softcap);
-  else
-    hipLaunchKernelGGL((masked_attn_rows_kernel<float>), dim3(T), dim3(256), lds, s, (const float*)q, (const float*)kc,
-                       (const float*)vc, block_tables, maxb, row_seg, seg_row0, seg_pos0, sink, gate, gs, (float*)out, H,
-                       G, D, V, BS, chunk, window, keep_first, scale, softcap);
+#define K8S_ROWS(TA, TO)                                                                                             \
+  hipLaunchKernelGGL((masked_attn_rows_kernel<TA, TO>), dim3(T), dim3(256), lds, s, (const TA*)q, (const TA*)kc,    \
+                     (const TA*)vc, block_tables, maxb, row_seg, seg_row0, seg_pos0, sink, gate, gs, (TO*)out, HQ, G, \
+                     D, V, BS, chunk, window, keep_first, scale, softcap, maps)
+  if (dt == 0 && out_f32) {
+    K8S_ROWS(uint16_t, float);
+  } else if (dt == 0) {
+    K8S_ROWS(uint16_t, uint16_t);
+  } else {
+    K8S_ROWS(float, float);
+  }
+#undef K8S_ROWS
   return (int)hipGetLastError();
 }
 
@@ -597,9 +650,10 @@ K8S_API int k8s_masked_attn_mfma_ok(int H, int G, int D, int V) {
 K8S_API int k8s_masked_attn_mfma(const void* q, const void* kc, const void* vt, const int* block_tables, int maxb,
                                  const int* items, int n_items, const float* sink, const float* gate, int gs, void* out,
                                  int H, int G, int D, int V, int BS, int chunk, int window, int keep_first, float scale,
-                                 float softcap, hipStream_t s, int part_blocks, int n_parts, float* pml, float* po) {
+                                 float softcap, hipStream_t s, int part_blocks, int n_parts, float* pml, float* po,
+                                 int maps, int out_f32) {
   if (n_items <= 0) return 0;
-  if (!k8s_masked_attn_mfma_ok(H, G, D, V) || BS % 32 || chunk < 0 || window < 0 || keep_first < 0)
+  if (!k8s_masked_attn_mfma_ok(H, G, D, V) || BS % 32 || chunk < 0 || window < 0 || keep_first < 0 || maps < 1)
     return (int)hipErrorInvalidValue;
   if (n_parts > 1 && (part_blocks < 1 || !pml || !po)) return (int)hipErrorInvalidValue;
   MaskArgs a;
@@ -613,9 +667,11 @@ K8S_API int k8s_masked_attn_mfma(const void* q, const void* kc, const void* vt, 
   a.sink = sink;
   a.gate = gate;
   a.gs = gs;
-  a.out = (uint16_t*)out;
-  a.H = H;
+  a.out = out_f32 ? nullptr : (uint16_t*)out;
+  a.out32 = out_f32 ? (float*)out : nullptr;
+  a.H = H * maps;
   a.G = G;
+  a.M = maps;
   a.BS = BS;
   a.chunk = chunk;
   a.window = window;

@@ -392,25 +392,33 @@ __global__ void __launch_bounds__(256) delta_carry_kernel(MatArgs p, const int* 
   }
 }
 
-// out[r][h] = u / sqrt(mean(u^2 over the head's V) + eps) * w * sigmoid(gate), u = o * mul[r][h] (mul optional):
-// one wave per (row, head).
+// out[r][h] = u / sqrt(mean(u^2 over the head's V) + eps) * w * sigmoid(gate) * oscale, u = o * mul[r][h] (mul
+// optional): one wave per (row, head).  w and gate are optional (absent: 1).
 // w is indexed h * wh + c: wh = V for a weight of all heads' size, 0 for one shared by the heads.
+// sub: o holds two results per head, [r][h][2][V], and u = o[.][0] - lam o[.][1] (two score maps joined).
 template <typename TA>
 __global__ void __launch_bounds__(256) head_norm_sigmoid_kernel(const float* __restrict__ o, const float* __restrict__ gate,
                                                                 int gs, const float* __restrict__ w, int wh,
                                                                 TA* __restrict__ out, int n_rh, int H, int V, float eps,
-                                                                const float* __restrict__ mul) {
+                                                                const float* __restrict__ mul, int sub, float lam,
+                                                                float oscale) {
   const int rh = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (rh >= n_rh) return;
   const int r = rh / H, h = rh - r * H;
-  const float* op = o + (size_t)rh * V;
+  const float* op = o + (size_t)rh * V * (sub ? 2 : 1);
   const float mu = mul ? mul[rh] : 1.f;
   float ss = 0.f;
-  for (int c = lane; c < V; c += 64) ss = fmaf(op[c] * mu, op[c] * mu, ss);
-  const float rn = mu / sqrtf(wave_sum(ss) / (float)V + eps);
-  const float* g = gate + (size_t)r * gs + (size_t)h * V;
-  const float* wp = w + (size_t)h * wh;
-  for (int c = lane; c < V; c += 64) stx(out, (size_t)rh * V + c, op[c] * rn * wp[c] * sigmoid_f(g[c]));
+  for (int c = lane; c < V; c += 64) {
+    const float u = (sub ? op[c] - lam * op[V + c] : op[c]) * mu;
+    ss = fmaf(u, u, ss);
+  }
+  const float rn = mu * oscale / sqrtf(wave_sum(ss) / (float)V + eps);
+  const float* g = gate ? gate + (size_t)r * gs + (size_t)h * V : nullptr;
+  const float* wp = w ? w + (size_t)h * wh : nullptr;
+  for (int c = lane; c < V; c += 64) {
+    const float u = sub ? op[c] - lam * op[V + c] : op[c];
+    stx(out, (size_t)rh * V + c, u * rn * (wp ? wp[c] : 1.f) * (g ? sigmoid_f(g[c]) : 1.f));
+  }
 }
 
 template <int DPT, int KIND, int MODE, bool FULL, typename TA>
@@ -542,14 +550,15 @@ K8S_API int k8s_matrix_memory(const float* x, int xs, const float* gate_bias, fl
 
 // mul (optional) [T][H]: o is multiplied by it before the norm
 K8S_API int k8s_head_norm_gate(const float* o, const float* gate, int gs, const float* w, int wh, void* out, int T,
-                               int H, int V, float eps, int odt, hipStream_t s, const float* mul) {
+                               int H, int V, float eps, int odt, hipStream_t s, const float* mul, int sub, float lam,
+                               float oscale) {
   if (T <= 0) return 0;
   const int n_rh = T * H;
   if (odt == 0)
     hipLaunchKernelGGL((head_norm_sigmoid_kernel<uint16_t>), dim3((n_rh + 3) / 4), dim3(256), 0, s, o, gate, gs, w, wh,
-                       (uint16_t*)out, n_rh, H, V, eps, mul);
+                       (uint16_t*)out, n_rh, H, V, eps, mul, sub, lam, oscale);
   else
     hipLaunchKernelGGL((head_norm_sigmoid_kernel<float>), dim3((n_rh + 3) / 4), dim3(256), 0, s, o, gate, gs, w, wh,
-                       (float*)out, n_rh, H, V, eps, mul);
+                       (float*)out, n_rh, H, V, eps, mul, sub, lam, oscale);
   return (int)hipGetLastError();
 }

@@ -266,6 +266,101 @@ __global__ void __launch_bounds__(128) scan_carry_kernel(const float* __restrict
     if (n < N) st[n] = S[n];
 }
 
+// State-space recurrence with ONE decay per head and token (the scalar-decay form of the selective scan), one
+// thread per channel c = h P + p of head h, the channel's N states in registers:
+//   dt = softplus(dtp[r][h] + dt_bias[h]);  a = exp(-rate[h] dt);  S[n] <- a S[n] + dt x[r][c] B[r][g][n];
+//   y[r][c] = (sum_n S[n] C[r][g][n] + D[h] x[r][c]) * silu(z[r][c]),   g = h / hpg (heads per B / C group).
+// x (row stride xs), bc rows (stride bs: B [G][N] | C [G][N]) and z (stride zs) have type TA; dtp (stride dts) is
+// fp32; y [T][C] fp32.  state [slots][C][N].  EX picks the exponentials (DecayExp).  MODE 0 / 1 / 2 and the chunk
+// arrays as in selective_scan_kernel; a chunk's decay is exp(-rate * sum dt), kept per (chunk, channel) in csd.
+template <int NMAX, int MODE, typename TA, typename EX>
+__global__ void __launch_bounds__(128) ssd_scan_kernel(const TA* __restrict__ x, int xs, const TA* __restrict__ bc, int bs,
+                                                       const float* __restrict__ dtp, int dts,
+                                                       const float* __restrict__ dt_bias, const float* __restrict__ rate,
+                                                       const float* __restrict__ Dp, const TA* __restrict__ z, int zs,
+                                                       float* __restrict__ state, const int* __restrict__ seg_row0,
+                                                       const int* __restrict__ seg_pos0, const int* __restrict__ seg_slot,
+                                                       float* __restrict__ y, int C, int N, int P, int hpg, int G,
+                                                       const int* __restrict__ chunks, float* __restrict__ cs,
+                                                       float* __restrict__ csd) {
+  const int it = blockIdx.x, c = blockIdx.y * 128 + threadIdx.x;
+  if (c >= C) return;
+  int r0, r1;
+  bool fresh;
+  float* st;
+  if (MODE == 0) {
+    r0 = seg_row0[it];
+    r1 = seg_row0[it + 1];
+    fresh = seg_pos0[it] == 0;
+    st = state + ((size_t)seg_slot[it] * C + c) * N;
+  } else {
+    r0 = chunks[it * 4 + 1];
+    r1 = r0 + chunks[it * 4 + 2];
+    fresh = MODE == 1;
+    st = cs + ((size_t)it * C + c) * N;
+  }
+  const int h = c / P, g = h / hpg;
+  float S[NMAX];
+#pragma unroll
+  for (int n = 0; n < NMAX; ++n) S[n] = (n < N && !fresh) ? st[n] : 0.f;
+  const float Dc = Dp[h], bias = dt_bias[h], nrate = -rate[h] * EX::kPre;
+  float sd = 0.f;
+  for (int r = r0; r < r1; ++r) {
+    const float dt = EX::softplus(dtp[(size_t)r * dts + h] + bias);
+    const float a = EX::f(dt * nrate);
+    const float xv = ldm(x, (size_t)r * xs + c);
+    const float dx = dt * xv;
+    const TA* Bp = bc + (size_t)r * bs + (size_t)g * N;
+    const TA* Cp = Bp + (size_t)G * N;
+    float acc = 0.f;
+    sd += dt;
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n)
+      if (n < N) {
+        S[n] = fmaf(a, S[n], dx * ldm(Bp, n));
+        if (MODE != 1) acc = fmaf(S[n], ldm(Cp, n), acc);
+      }
+    if (MODE != 1) y[(size_t)r * C + c] = (acc + Dc * xv) * EX::silu(ldm(z, (size_t)r * zs + c));
+  }
+  if (MODE != 2) {
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n)
+      if (n < N) st[n] = S[n];
+  }
+  if (MODE == 1) csd[(size_t)it * C + c] = sd;
+}
+
+// Between the two chunk passes of ssd_scan_kernel: every chunk's end-from-zero state becomes its START state,
+// the segment's final state goes to the slot (scan_carry_kernel with one decay per head).
+template <int NMAX>
+__global__ void __launch_bounds__(128) ssd_carry_kernel(const float* __restrict__ rate, float* __restrict__ state,
+                                                        const int* __restrict__ seg_pos0, const int* __restrict__ seg_slot,
+                                                        const int* __restrict__ seg_chunk0, float* __restrict__ cs,
+                                                        const float* __restrict__ csd, int C, int N, int P) {
+  const int sg = blockIdx.x, c = blockIdx.y * 128 + threadIdx.x;
+  if (c >= C) return;
+  float* st = state + ((size_t)seg_slot[sg] * C + c) * N;
+  const bool fresh = seg_pos0[sg] == 0;
+  const float nrate = -rate[c / P];
+  float S[NMAX];
+#pragma unroll
+  for (int n = 0; n < NMAX; ++n) S[n] = (n < N && !fresh) ? st[n] : 0.f;
+  for (int k = seg_chunk0[sg]; k < seg_chunk0[sg + 1]; ++k) {
+    float* ck = cs + ((size_t)k * C + c) * N;
+    const float a = expf(csd[(size_t)k * C + c] * nrate);
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n)
+      if (n < N) {
+        const float loc = ck[n];
+        ck[n] = S[n];
+        S[n] = fmaf(a, S[n], loc);
+      }
+  }
+#pragma unroll
+  for (int n = 0; n < NMAX; ++n)
+    if (n < N) st[n] = S[n];
+}
+
 // Retention in three kernels.  Rows of qkvg (fp32, stride qs): q [H][D] | k [H][D] | v [H][V] | g [H][V].
 //   1. retention_rope_kernel (one workgroup per token, in place): q and k are rotated on their first
 //      `rot` entries (entry i with i + rot / 2; angle = pos * base^(-2 i / rot), formed in double) and k is
@@ -516,6 +611,49 @@ K8S_API int k8s_selective_scan(const void* xc, int dt, const float* dtp, const f
   }
 #undef K8S_SCAN
 #undef K8S_SCAN_M
+  return (int)hipGetLastError();
+}
+
+// fast != 0: the hardware exponentials (DecayExp<uint16_t>), else expf / log1pf.  dt: the type of x, bc and z.
+K8S_API int k8s_ssd_scan(const void* x, int xs, const void* bc, int bs, int dt, const float* dtp, int dts,
+                         const float* dt_bias, const float* rate, const float* D, const void* z, int zs, float* state,
+                         const int* seg_row0, const int* seg_pos0, const int* seg_slot, float* y, int n_seg, int H,
+                         int P, int G, int N, int T, int fast, hipStream_t s, const int* chunks, int n_chunks,
+                         const int* seg_chunk0, float* cs, float* csd) {
+  if (T <= 0 || n_seg <= 0) return 0;
+  if (N < 1 || N > 128 || H < 1 || P < 1 || G < 1 || H % G) return (int)hipErrorInvalidValue;
+  const int C = H * P, cb = (C + 127) / 128, hpg = H / G;
+#define K8S_SSD_E(NM, MODE, items, EX)                                                                            \
+  K8S_MDT(dt, hipLaunchKernelGGL((ssd_scan_kernel<NM, MODE, TA, EX>), dim3(items, cb), dim3(128), 0, s,           \
+                                 (const TA*)x, xs, (const TA*)bc, bs, dtp, dts, dt_bias, rate, D, (const TA*)z,   \
+                                 zs, state, seg_row0, seg_pos0, seg_slot, y, C, N, P, hpg, G, chunks, cs, csd))
+#define K8S_SSD_M(NM, MODE, items)                \
+  if (fast) {                                     \
+    K8S_SSD_E(NM, MODE, items, DecayExp<uint16_t>) \
+  } else {                                        \
+    K8S_SSD_E(NM, MODE, items, DecayExp<float>)   \
+  }
+#define K8S_SSD(NM)                                                                                             \
+  if (chunks == nullptr) {                                                                                      \
+    K8S_SSD_M(NM, 0, n_seg)                                                                                     \
+  } else {                                                                                                      \
+    K8S_SSD_M(NM, 1, n_chunks)                                                                                  \
+    hipLaunchKernelGGL((ssd_carry_kernel<NM>), dim3(n_seg, cb), dim3(128), 0, s, rate, state, seg_pos0, seg_slot, \
+                       seg_chunk0, cs, csd, C, N, P);                                                           \
+    K8S_SSD_M(NM, 2, n_chunks)                                                                                  \
+  }
+  if (N <= 16) {
+    K8S_SSD(16)
+  } else if (N <= 32) {
+    K8S_SSD(32)
+  } else if (N <= 64) {
+    K8S_SSD(64)
+  } else {
+    K8S_SSD(128)
+  }
+#undef K8S_SSD
+#undef K8S_SSD_M
+#undef K8S_SSD_E
   return (int)hipGetLastError();
 }
 

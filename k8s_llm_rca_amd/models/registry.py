@@ -6,8 +6,9 @@ checkpoint folder's config.json.
 * ``zasapel``             -- :class:`~.zasapel.ZasapelModel` (config.json with ``"architecture": "Zasapel"``)
 * ``ligipel``             -- :class:`~.ligipel.LigipelModel` (config.json with ``"architecture": "Ligipel"``)
 * ``lizesun``             -- :class:`~.lizesun.LizesunModel` (config.json with ``"architecture": "Lizesun"``)
+* ``pumozen``             -- :class:`~.pumozen.PumozenModel` (config.json with ``"architecture": "Pumozen"``)
 
-The last three describe their layers one by one in config.json (``OWN_CONFIG``): their
+The last four describe their layers one by one in config.json (``OWN_CONFIG``): their
 configuration objects are built from it, not from a preset with overrides.
 """
 from __future__ import annotations
@@ -21,7 +22,7 @@ from . import config as C
 
 # architectures whose config.json lists the layers (``"architecture": <name>``): module, model class
 OWN_CONFIG = {"zasapel": ("zasapel", "ZasapelModel"), "ligipel": ("ligipel", "LigipelModel"),
-              "lizesun": ("lizesun", "LizesunModel")}
+              "lizesun": ("lizesun", "LizesunModel"), "pumozen": ("pumozen", "PumozenModel")}
 
 
 def _module(arch: str):

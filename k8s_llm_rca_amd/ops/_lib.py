@@ -93,13 +93,15 @@ _SIGS = {
     "k8s_latent_attn_rows": [P, P, P, I, P, P, P, P, I, P, I, I, I, I, I, F, I, P],
     "k8s_polynorm": [P, P, P, I, I, F, I, P],
     "k8s_glu_clamp": [P, P, I, I, F, F, F, I, P],
-    "k8s_router": [P, P, I, I, I, I, I, I, P, P, I, P, P, F],
+    "k8s_router": [P, P, I, I, I, I, I, I, P, P, I, P, P, F, I, P, F],
     "k8s_moe_gather": [P, P, P, P, I, I, I, I, P],
     "k8s_moe_combine_f32": [P, P, P, P, I, I, I, I, P],
     "k8s_grouped_any": [P, P, P, P, I, I, I, I, I, P],
     "k8s_layernorm": [P, P, P, P, I, I, F, I, P],
     "k8s_embed_ln": [P, P, I, P, P, P, P, P, P, I, I, I, F, P],
-    "k8s_ln_residual": [P, P, P, I, P, P, P, P, P, P, P, P, I, I, I, F, P],
+    "k8s_ln_residual": [P, P, P, I, P, P, P, P, P, P, P, P, I, I, I, F, P, I, P, I],
+    "k8s_embed_rows": [P, P, I, P, P, I, I, I, P],
+    "k8s_token_gate": [P, P, P, I, I, I, P, I, I, I, P],
     "k8s_depth_mix_ln": [P, I, I, P, P, I, P, P, P, P, I, I, F, P],
     "k8s_softcap": [P, ctypes.c_long, F, F, P],
     "k8s_short_conv": [P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P, P, I],
@@ -112,13 +114,14 @@ _SIGS = {
     "k8s_add_dyt": [P, P, F, P, F, F, P, P, P, I, I, I, P],
     "k8s_embed_scale_dyt": [P, P, I, F, P, F, P, P, P, I, I, I, P],
     "k8s_relu_sq": [P, P, ctypes.c_long, I, P],
-    "k8s_attn_prep": [P, I, P, I, I, I, I, P, P, P, P, P, I, P, I, I, P, P, F, I, F, F, P, P, I, P],
-    "k8s_masked_attn_rows": [P, P, P, P, I, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, I, F, F, I, P],
+    "k8s_attn_prep": [P, I, P, I, I, I, I, P, P, P, P, P, I, P, I, I, P, P, F, I, F, F, P, P, I, P, I, F, I],
+    "k8s_masked_attn_rows": [P, P, P, P, I, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, I, F, F, I, P, I, I],
     "k8s_masked_attn_mfma_ok": [I, I, I, I],
-    "k8s_masked_attn_mfma": [P, P, P, P, I, P, I, P, P, I, P, I, I, I, I, I, I, I, I, F, F, P, I, I, P, P],
+    "k8s_masked_attn_mfma": [P, P, P, P, I, P, I, P, P, I, P, I, I, I, I, I, I, I, I, F, F, P, I, I, P, P, I, I],
     "k8s_gated_delta": [P, I, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, F, P, P, I, P, P, P],
     "k8s_matrix_memory": [P, I, P, F, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, P, P, I, P, P, P, P],
-    "k8s_head_norm_gate": [P, P, I, P, I, P, I, I, I, F, I, P, P],
+    "k8s_head_norm_gate": [P, P, I, P, I, P, I, I, I, F, I, P, P, I, F, F],
+    "k8s_ssd_scan": [P, I, P, I, I, P, I, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, P, P, I, P, P, P],
     "k8s_walks": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P, P, P, P],
 }
 # entry points whose C return type is not int

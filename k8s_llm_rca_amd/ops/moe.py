@@ -159,23 +159,28 @@ def _dt(t: torch.dtype) -> int:
 
 def route_direct(h: torch.Tensor, w_router: torch.Tensor, k: int, scoring: str = "sigmoid",
                  renorm: bool = False, choice_bias: Optional[torch.Tensor] = None,
-                 renorm_eps: float = 0.0) -> Tuple[torch.Tensor, torch.Tensor]:
+                 renorm_eps: float = 0.0, scale: float = 1.0, extra_rows: int = 0):
     """Router straight from the hidden rows: fp32 logits ``h @ w_router.T``, scores by ``scoring``
     ("sigmoid" or "softmax"), the ``k`` largest (ties: lowest index), renormalised only with
-    ``renorm`` (divided by their sum + ``renorm_eps``).  With ``choice_bias`` (fp32 [E]) the experts
-    are chosen by score + bias while the weights are the plain scores.
-    Returns (weights fp32 [T, k], ids int32 [T, k])."""
+    ``renorm`` (divided by their sum + ``renorm_eps``), then times ``scale``.  With ``choice_bias`` (fp32 [E])
+    the experts are chosen by score + bias while the weights are the plain scores.
+    Returns (weights fp32 [T, k], ids int32 [T, k]).  With ``extra_rows`` = X the last X rows of ``w_router``
+    are not experts: their fp32 logits are returned as a third result [T, X] (gates that read the same rows)."""
     T, W = h.shape
-    E = w_router.shape[0]
+    X = int(extra_rows)
+    E = w_router.shape[0] - X
     if use_hip(h):
         assert h.is_contiguous() and w_router.is_contiguous() and h.dtype == w_router.dtype
         w = torch.empty(T, k, dtype=torch.float32, device=h.device)
         ids = torch.empty(T, k, dtype=torch.int32, device=h.device)
+        extra = torch.empty(T, X, dtype=torch.float32, device=h.device) if X else None
         check(lib().k8s_router(ptr(h), ptr(w_router), T, W, E, k, 0 if scoring == "sigmoid" else 1, int(renorm),
-                               ptr(w), ptr(ids), _dt(h.dtype), stream_ptr(h), ptr(choice_bias), float(renorm_eps)),
-              "router")
-        return w, ids
+                               ptr(w), ptr(ids), _dt(h.dtype), stream_ptr(h), ptr(choice_bias), float(renorm_eps),
+                               X, ptr(extra), float(scale)), "router")
+        return (w, ids, extra) if X else (w, ids)
     z = h.float() @ w_router.float().t()
+    extra = z[:, E:].contiguous()
+    z = z[:, :E]
     s = torch.sigmoid(z) if scoring == "sigmoid" else torch.softmax(z, -1)
     # stable descending sort: equal scores keep the lower expert first
     c = s if choice_bias is None else s + choice_bias.float()
@@ -183,7 +188,9 @@ def route_direct(h: torch.Tensor, w_router: torch.Tensor, k: int, scoring: str =
     w = torch.gather(s, 1, order)
     if renorm:
         w = w / (w.sum(-1, keepdim=True) + renorm_eps)
-    return w, order.int()
+    if scale != 1.0:
+        w = w * scale
+    return (w, order.int(), extra) if X else (w, order.int())
 
 
 def gather_rows(h: torch.Tensor, order: torch.Tensor, k: int, w: Optional[torch.Tensor] = None) -> torch.Tensor:

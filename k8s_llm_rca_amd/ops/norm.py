@@ -149,24 +149,35 @@ def embed_layernorm(ids: torch.Tensor, embed: torch.Tensor, w: torch.Tensor, b: 
     return h
 
 
-def ln_residual(src: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float,
+def ln_residual(src: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], eps: float,
                 dst: torch.Tensor, y2: Optional[torch.Tensor] = None, merge: Optional[str] = None,
                 mw: Optional[tuple] = None, nw: Optional[torch.Tensor] = None, nb: Optional[torch.Tensor] = None,
-                out_dtype=None) -> Optional[torch.Tensor]:
+                out_dtype=None, kind: str = "layer", row_gate: Optional[torch.Tensor] = None,
+                cast: bool = False) -> Optional[torch.Tensor]:
     """``dst = src + LN(u; w, b)`` on fp32 rows (``dst`` may be ``src``), where ``u`` is the sublayer
     output ``y``, or two outputs joined: ``merge="sum"``: ``y + y2``; ``merge="rms"``:
-    ``(unit_rms(y) mw[0] + unit_rms(y2) mw[1]) / 2``.  With ``nw, nb`` also returns ``LN(dst; nw, nb)`` as
-    activations (the next sublayer's input norm, same pass)."""
+    ``(unit_rms(y) mw[0] + unit_rms(y2) mw[1]) / 2``; ``merge="gated"``: ``y + sigmoid(row_gate) y2`` with one gate
+    logit per row (``row_gate`` [T] or a column [T, 1] of a wider fp32 matrix).  ``kind="rms"``: the norm is
+    ``u / sqrt(mean(u^2) + eps) * w`` instead (``b`` None).  With ``nw, nb`` also returns ``LN(dst; nw, nb)`` as
+    activations (the next sublayer's input norm, same pass); with ``cast`` the new rows themselves as
+    activations (the next sublayer reads the residual as it is)."""
     T, W = src.shape
-    h = torch.empty(T, W, dtype=out_dtype, device=src.device) if nw is not None else None
-    mode = {None: 0, "rms": 1, "sum": 2}[merge if y2 is not None else None]
+    assert not (cast and nw is not None)
+    h = torch.empty(T, W, dtype=out_dtype, device=src.device) if (nw is not None or cast) else None
+    mode = {None: 0, "rms": 1, "sum": 2, "gated": 3}[merge if y2 is not None else None]
+    knd = {"layer": 0, "rms": 1}[kind]
     if use_hip(src):
         for t in (src, y, dst) + ((y2,) if y2 is not None else ()):
             assert t.dtype == torch.float32 and t.is_contiguous() and t.shape == (T, W)
         wl, wr = mw if mode == 1 else (None, None)
+        rgs = 0
+        if mode == 3:
+            assert row_gate.dtype == torch.float32 and row_gate.shape[0] == T and row_gate.numel() == T
+            rgs = row_gate.stride(0)
         check(lib().k8s_ln_residual(ptr(src), ptr(y), ptr(y2), mode, ptr(wl), ptr(wr), ptr(w), ptr(b), ptr(dst),
                                     ptr(nw), ptr(nb), ptr(h), _odt(out_dtype) if h is not None else 1, T, W,
-                                    float(eps), stream_ptr(src)), "ln_residual")
+                                    float(eps), stream_ptr(src), knd, ptr(row_gate) if mode == 3 else 0, rgs),
+              "ln_residual")
         return h
     if mode == 1:
         def unit(v):
@@ -174,12 +185,51 @@ def ln_residual(src: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: torch.Te
         u = 0.5 * (unit(y) * mw[0] + unit(y2) * mw[1])
     elif mode == 2:
         u = y + y2
+    elif mode == 3:
+        u = y + torch.sigmoid(row_gate.reshape(T, 1)) * y2
     else:
         u = y
-    dst.copy_(src + _ln(u, w, b, eps))
-    if h is not None:
+    if knd == 1:
+        dst.copy_(src + u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w)
+    else:
+        dst.copy_(src + _ln(u, w, b, eps))
+    if nw is not None:
         h.copy_(_ln(dst, nw, nb, eps).to(out_dtype))
+    elif cast:
+        h.copy_(dst.to(out_dtype))
     return h
+
+
+def embed_rows(ids: torch.Tensor, embed: torch.Tensor, x_out: torch.Tensor, out_dtype=None) -> Optional[torch.Tensor]:
+    """``x_out = embed[ids]`` (fp32); with ``out_dtype`` also returns the rows as activations of that type."""
+    T, W = ids.shape[0], embed.shape[1]
+    h = torch.empty(T, W, dtype=out_dtype, device=embed.device) if out_dtype is not None else None
+    if use_hip(embed):
+        assert x_out.dtype == torch.float32 and x_out.is_contiguous() and x_out.shape == (T, W)
+        assert embed.is_contiguous() and ids.dtype == torch.int32
+        check(lib().k8s_embed_rows(ptr(ids), ptr(embed), _odt(embed.dtype), ptr(x_out), ptr(h),
+                                   _odt(out_dtype) if h is not None else 1, T, W, stream_ptr(embed)), "embed_rows")
+        return h
+    x_out.copy_(embed[ids.long()].float())
+    if h is not None:
+        h.copy_(x_out.to(out_dtype))
+    return h
+
+
+def token_gate(a: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: int, out_dtype) -> torch.Tensor:
+    """``gelu_tanh(a) * table[ids, col0 : col0 + n]`` for fp32 ``a`` [T, n] as activations: a per-token input looked up
+    by token id and gated by a projection of the hidden row (``gelu_tanh(z) = z / 2 (1 + tanh(sqrt(2 / pi)
+    (z + 0.044715 z^3)))``)."""
+    T, n = a.shape
+    out = torch.empty(T, n, dtype=out_dtype, device=a.device)
+    if use_hip(a):
+        assert a.dtype == torch.float32 and a.is_contiguous() and table.is_contiguous() and ids.dtype == torch.int32
+        check(lib().k8s_token_gate(ptr(a), ptr(ids), ptr(table), _odt(table.dtype), table.shape[1], int(col0),
+                                   ptr(out), _odt(out_dtype), T, n, stream_ptr(a)), "token_gate")
+        return out
+    g = torch.nn.functional.gelu(a, approximate="tanh")
+    out.copy_((g * table[ids.long(), col0:col0 + n].float()).to(out_dtype))
+    return out
 
 
 def depth_mix_ln(stack: torch.Tensor, n: int, coef: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float,

@@ -438,6 +438,57 @@ def selective_scan(xc: torch.Tensor, dtp: torch.Tensor, dt_bias: torch.Tensor, d
     return y
 
 
+def ssd_scan(x: torch.Tensor, bc: torch.Tensor, dtp: torch.Tensor, dt_bias: torch.Tensor, rate: torch.Tensor,
+             D: torch.Tensor, z: torch.Tensor, H: int, P: int, G: int, N: int, state: torch.Tensor, seg: SegMeta,
+             fast_exp: bool = False) -> torch.Tensor:
+    """State-space recurrence with one decay per head and token (state-space duality), fp32.  Head h of ``H`` owns
+    the channels ``h P .. h P + P - 1`` of ``x`` [T, H P] and reads B / C group ``h // (H // G)`` of ``bc`` [T, 2 G N]
+    = (B [G, N] | C [G, N]):  ``dt = softplus(dtp[:, h] + dt_bias[h])``;  ``S <- exp(-rate[h] dt) S + dt B x^T``
+    (``S`` [N, P] per head);  ``y = (S^T C + D[h] x) * silu(z)``.  ``x``, ``bc``, ``z`` are activations of one type and
+    may be column slices; ``dtp`` [T, H] fp32 (row stride free).  ``state`` [slots, H P, N] fp32 is read (past
+    position 0) and advanced.  Returns y [T, H P] fp32.  ``fast_exp``: the hardware exponentials (relative error
+    about 1e-6) instead of ``expf`` / ``log1pf``."""
+    T, C = x.shape
+    y = torch.empty(T, C, dtype=torch.float32, device=x.device)
+    if use_hip(x):
+        assert C == H * P and H % G == 0 and 1 <= N <= 128 and bc.shape[1] == 2 * G * N
+        assert x.stride(1) == bc.stride(1) == z.stride(1) == dtp.stride(1) == 1 and x.dtype == bc.dtype == z.dtype
+        assert dtp.dtype == torch.float32 and dtp.shape[1] == H and z.shape[1] == C
+        assert dt_bias.dtype == rate.dtype == D.dtype == torch.float32 and dt_bias.numel() == rate.numel() == D.numel() == H
+        assert state.is_contiguous() and state.shape[1:] == (C, N)
+        # long portions: chunks in parallel (end states from zero + the sum of step sizes, a carry over the
+        # chunks, the chunks again from their start states); short ones, and steps whose sequences x channels
+        # already fill the chip, token by token
+        cr = seg.chunk_ranges(SSM_CHUNK, 2 * SSM_CHUNK) if seg.n_seg * C < SEQ_FILL_LANES else None
+        chunks, c0, cs, csd, nch = None, None, None, None, 0
+        if cr is not None:
+            chunks, c0 = cr
+            nch = chunks.shape[0]
+            cs = scratch(nch * C * N, torch.float32, x.device)
+            csd = scratch(nch * C, torch.float32, x.device)
+        check(lib().k8s_ssd_scan(ptr(x), x.stride(0), ptr(bc), bc.stride(0), _dt(x.dtype), ptr(dtp), dtp.stride(0),
+                                 ptr(dt_bias), ptr(rate), ptr(D), ptr(z), z.stride(0), ptr(state), ptr(seg.seg_row0),
+                                 ptr(seg.seg_pos0), ptr(seg.seg_slot), ptr(y), seg.n_seg, H, P, G, N, T,
+                                 int(fast_exp), stream_ptr(x), ptr(chunks), nch, ptr(c0), ptr(cs), ptr(csd)),
+              "ssd_scan")
+        return y
+    dt = torch.nn.functional.softplus(dtp.float() + dt_bias)                 # [T, H]
+    dec = torch.exp(-rate * dt)
+    xf, zf = x.float().view(T, H, P), z.float()
+    rep = H // G
+    Bm = bc[:, :G * N].float().view(T, G, N).repeat_interleave(rep, 1)      # [T, H, N]
+    Cm = bc[:, G * N:].float().view(T, G, N).repeat_interleave(rep, 1)
+    for s in range(seg.n_seg):
+        a, e, p0, sl = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s], seg.slot_host[s]
+        S = state[sl].view(H, P, N).clone() if p0 > 0 else torch.zeros(H, P, N)
+        for r in range(a, e):
+            S = dec[r][:, None, None] * S + (dt[r][:, None] * xf[r])[:, :, None] * Bm[r][:, None, :]
+            o = torch.einsum("hpn,hn->hp", S, Cm[r]) + D[:, None] * xf[r]
+            y[r] = o.reshape(-1) * torch.nn.functional.silu(zf[r])
+        state[sl] = S.reshape(C, N)
+    return y
+
+
 def retention(qkvg: torch.Tensor, H: int, D: int, V: int, decay: torch.Tensor, rot_dims: int, rot_base: float,
               state: torch.Tensor, seg: SegMeta, positions: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
     """Retention per head, fp32: rows of ``qkvg`` [T, 2HD + 2HV] fp32 = (q | k | v | g).  q and k are
@@ -595,39 +646,56 @@ def window_attention(qkv: torch.Tensor, H: int, G: int, D: int, V: int, kc: torc
 # ------------------------------------------------------------------ masked softmax attention with a prepared q / k,
 # and matrix-state recurrences (csrc/kernels/masked_attn.hip, matrix_mem.hip)
 def attn_prep(qkv: torch.Tensor, bias: Optional[torch.Tensor], H: int, G: int, D: int, V: int,
-              positions: torch.Tensor, slots: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, out_dtype,
-              norm: bool = False, q_w: Optional[torch.Tensor] = None, k_w: Optional[torch.Tensor] = None,
+              positions: torch.Tensor, slots: torch.Tensor, kc: Optional[torch.Tensor], vc: Optional[torch.Tensor],
+              out_dtype, norm=False, q_w: Optional[torch.Tensor] = None, k_w: Optional[torch.Tensor] = None,
               eps: float = 0.0, rot_dims: int = 0, rot_base: float = 10000.0, lam: float = 0.0,
               v_other: Optional[torch.Tensor] = None, v_keep: Optional[torch.Tensor] = None,
-              vt: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Between the joint projection and attention, one pass over the fp32 rows of ``qkv`` [T, H D + G D + G V]
-    = (q | k | v):  add ``bias`` (fp32, same width, optional);  rotate q and k on their first ``rot_dims``
-    entries per head (entry i paired with i + rot_dims / 2, angle ``pos * rot_base^(-2 i / rot_dims)``);  with
-    ``norm`` divide every q and k head by its root mean square (``eps`` inside the root) and multiply by
-    ``q_w`` / ``k_w`` [D] where given;  ``v_keep`` [T, G V] fp32 receives the values as projected;  with
-    ``v_other`` the values become ``(1 - lam) v + lam v_other``.  k and v go to the pages ``kc`` [pages, BS, G D] /
-    ``vc`` [pages, BS, G V] at ``slots`` (and v to the transposed twin ``vt`` when given); q is returned
-    [T, H D] as activations."""
+              vt: Optional[torch.Tensor] = None, maps: int = 1, v_is_k: bool = False,
+              q_temp: Optional[Tuple[float, int]] = None) -> torch.Tensor:
+    """Between the joint projection and attention, one pass over the fp32 rows of ``qkv`` [T, H M D + G M D + G V]
+    = (q | k | v) with ``M = maps`` score maps per head (q and k laid out [head][map][D]):  add ``bias`` (fp32, same
+    width, optional);  rotate q and k on their first ``rot_dims`` entries per head (entry i paired with
+    i + rot_dims / 2, angle ``pos * rot_base^(-2 i / rot_dims)``);  with ``norm`` (True or "head") divide every q and k
+    head by its root mean square (``eps`` inside the root) and multiply by ``q_w`` / ``k_w`` [D] where given -- behind
+    the rotation;  with ``norm="all"`` divide q, and k, by the root mean square of the WHOLE projection and multiply by
+    ``q_w`` [H M D] / ``k_w`` [G M D] -- in front of the rotation;  with ``q_temp = (coef, every)`` multiply q by
+    ``1 + coef ln(floor((pos + 1) / every) + 1)``;  ``v_keep`` [T, G V] fp32 receives the values as projected;  with
+    ``v_other`` the values become ``(1 - lam) v + lam v_other``.  ``v_is_k``: there are no value columns, the values
+    are the keys as projected (before norm and rotation; V = M D).  k and v go to the pages ``kc`` [pages, BS, G M D] /
+    ``vc`` [pages, BS, G V] at ``slots`` (and v to the transposed twin ``vt`` when given); q is returned [T, H M D] as
+    activations.  ``G = 0``: only queries (a layer that reads another layer's pages)."""
     T = qkv.shape[0]
-    NQ, NK, NV = H * D, G * D, G * V
+    HQ, GK = H * maps, G * maps
+    NQ, NK, NV = HQ * D, GK * D, G * V
+    mode = {False: 0, None: 0, True: 1, "head": 1, "all": 2}[norm]
+    v_col = NQ if v_is_k else NQ + NK
+    assert not v_is_k or NV == NK
     q_out = torch.empty(T, NQ, dtype=out_dtype, device=qkv.device)
-    BS = kc.shape[1]
+    BS = kc.shape[1] if kc is not None else 1
+    tq_coef, tq_every = (float(q_temp[0]), int(q_temp[1])) if q_temp else (0.0, 0)
     if use_hip(qkv):
-        assert qkv.dtype == torch.float32 and qkv.stride(1) == 1 and qkv.shape[1] == NQ + NK + NV
-        assert kc.is_contiguous() and vc.is_contiguous() and kc.dtype == vc.dtype == out_dtype
-        assert kc.shape[-1] == NK and vc.shape[-1] == NV and rot_dims % 2 == 0 and 0 <= rot_dims <= D
-        for t in (bias, q_w, k_w):
-            assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+        assert qkv.dtype == torch.float32 and qkv.stride(1) == 1 and qkv.shape[1] == v_col + NV
+        if G:
+            assert kc.is_contiguous() and vc.is_contiguous() and kc.dtype == vc.dtype == out_dtype
+            assert kc.shape[-1] == NK and vc.shape[-1] == NV
+        assert rot_dims % 2 == 0 and 0 <= rot_dims <= D
+        for t, n in ((bias, v_col + NV), (q_w, NQ if mode == 2 else D), (k_w, NK if mode == 2 else D)):
+            assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n)
         for t in (v_other, v_keep):
             assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.shape == (T, NV))
         assert vt is None or (vt.is_contiguous() and vt.dtype == out_dtype and vt.shape[1:] == (NV, BS))
-        check(lib().k8s_attn_prep(ptr(qkv), qkv.stride(0), ptr(bias), H, G, D, V, ptr(positions), ptr(slots),
-                                  ptr(kc), ptr(vc), ptr(vt), BS, ptr(q_out), _dt(out_dtype), int(norm), ptr(q_w),
+        check(lib().k8s_attn_prep(ptr(qkv), qkv.stride(0), ptr(bias), HQ, GK, D, NV, ptr(positions), ptr(slots),
+                                  ptr(kc), ptr(vc), ptr(vt), BS, ptr(q_out), _dt(out_dtype), mode, ptr(q_w),
                                   ptr(k_w), float(eps), int(rot_dims), float(rot_base), float(lam), ptr(v_other),
-                                  ptr(v_keep), T, stream_ptr(qkv)), "attn_prep")
+                                  ptr(v_keep), T, stream_ptr(qkv), v_col, tq_coef, tq_every), "attn_prep")
         return q_out
     x = qkv + bias if bias is not None else qkv
-    q, k, v = x[:, :NQ].reshape(T, H, D), x[:, NQ:NQ + NK].reshape(T, G, D), x[:, NQ + NK:]
+    q, k, v = x[:, :NQ], x[:, NQ:NQ + NK], x[:, v_col:v_col + NV]
+    if mode == 2:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * (q_w if q_w is not None else 1.0)
+        if NK:
+            k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * (k_w if k_w is not None else 1.0)
+    q, k = q.reshape(T, HQ, D), k.reshape(T, GK, D)
     if rot_dims:
         half = rot_dims // 2
         f = torch.exp(-(2.0 * torch.arange(half, dtype=torch.float64) / rot_dims) * math.log(rot_base))
@@ -639,23 +707,27 @@ def attn_prep(qkv: torch.Tensor, bias: Optional[torch.Tensor], H: int, G: int, D
             return torch.cat([a * co - b * si, b * co + a * si, z[..., rot_dims:]], -1)
 
         q, k = rot(q), rot(k)
-    if norm:
+    if mode == 1:
         q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)
         k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
         if q_w is not None:
             q = q * q_w
         if k_w is not None:
             k = k * k_w
+    if tq_every:
+        temp = 1.0 + tq_coef * torch.log(torch.div(positions + 1, tq_every, rounding_mode="floor").float() + 1.0)
+        q = q * temp[:, None, None]
     if v_keep is not None:
         v_keep.copy_(v)
     if v_other is not None:
         v = (1.0 - lam) * v + lam * v_other
-    ok = slots >= 0
-    sl = slots[ok].long()
-    kc.view(-1, NK)[sl] = k.reshape(T, NK)[ok].to(kc.dtype)
-    vc.view(-1, NV)[sl] = v[ok].to(vc.dtype)
-    if vt is not None:
-        vt[sl // BS, :, sl % BS] = v[ok].to(vt.dtype)
+    if G:
+        ok = slots >= 0
+        sl = slots[ok].long()
+        kc.view(-1, NK)[sl] = k.reshape(T, NK)[ok].to(kc.dtype)
+        vc.view(-1, NV)[sl] = v[ok].to(vc.dtype)
+        if vt is not None:
+            vt[sl // BS, :, sl % BS] = v[ok].to(vt.dtype)
     q_out.copy_(q.reshape(T, NQ).to(out_dtype))
     return q_out
 
@@ -663,7 +735,7 @@ def attn_prep(qkv: torch.Tensor, bias: Optional[torch.Tensor], H: int, G: int, D
 def masked_attention(q: torch.Tensor, H: int, G: int, D: int, V: int, kc: torch.Tensor, vc: torch.Tensor,
                      seg: SegMeta, scale: float, softcap: float = 0.0, chunk: int = 0, window: int = 0,
                      keep_first: int = 0, sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
-                     vt: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     vt: Optional[torch.Tensor] = None, maps: int = 1, out_f32: bool = False) -> torch.Tensor:
     """Softmax attention of the rows' queries ``q`` [T, H D] over the paged keys and values (which already
     hold this step's rows), query head h reading key / value head ``h // (H // G)``.  Position i sees j <= i
     with, for ``chunk`` > 0, ``i // chunk == j // chunk`` and, for ``window`` > 0, ``i - j < window or j < keep_first``
@@ -671,16 +743,21 @@ def masked_attention(q: torch.Tensor, H: int, G: int, D: int, V: int, kc: torch.
     ``softcap`` > 0.  ``sink`` [H] fp32 adds ``exp(sink_h)`` to head h's denominator (no key, no value).  ``gate``
     [T, >= H] fp32 (row stride free): head h's output is multiplied by ``sigmoid(gate[t, h])``.
     Returns [T, H V].  With the transposed value pages ``vt`` (bf16, sizes of :func:`masked_mfma_ok`) the
-    matrix-core kernel runs."""
+    matrix-core kernel runs.
+    ``maps`` = M > 1: every head has M score maps -- ``q`` is [T, H M D] and the key pages [.., G M D], both laid out
+    [head][map][D]; map m of head h scores against key head ``(h // (H // G)) M + m``, has a softmax of its own and
+    applies it to value head ``h // (H // G)``; the result is [T, H M V], every map's by itself (``sink`` and ``gate``
+    then count H M).  ``out_f32``: the result in fp32 whatever the activation type."""
     T = q.shape[0]
     BS = kc.shape[1]
-    out = torch.empty(T, H * V, dtype=q.dtype, device=q.device)
+    HQ = H * maps
+    out = torch.empty(T, HQ * V, dtype=torch.float32 if out_f32 else q.dtype, device=q.device)
     if use_hip(q):
-        assert q.is_contiguous() and q.shape[1] == H * D and kc.is_contiguous() and vc.is_contiguous()
-        assert kc.dtype == vc.dtype == q.dtype and kc.shape[-1] == G * D and vc.shape[-1] == G * V and H % G == 0
+        assert q.is_contiguous() and q.shape[1] == HQ * D and kc.is_contiguous() and vc.is_contiguous()
+        assert kc.dtype == vc.dtype == q.dtype and kc.shape[-1] == G * maps * D and vc.shape[-1] == G * V and H % G == 0
         assert seg.block_tables.is_contiguous() and chunk >= 0 and window >= 0 and keep_first >= 0
-        assert sink is None or (sink.dtype == torch.float32 and sink.shape[0] == H)
-        assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.shape[1] >= H)
+        assert sink is None or (sink.dtype == torch.float32 and sink.shape[0] == HQ)
+        assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.shape[1] >= HQ)
         gs = gate.stride(0) if gate is not None else 0
         if vt is not None and masked_mfma_ok(H, G, D, V, q.dtype, q.device):
             assert vt.is_contiguous() and vt.shape[1:] == (G * V, BS) and BS % 32 == 0
@@ -699,36 +776,36 @@ def masked_attention(q: torch.Tensor, H: int, G: int, D: int, V: int, kc: torch.
                 pb = max(MASK_PART_BLOCKS, -(-nblk // MASK_MAX_PARTS))
                 n_parts = -(-nblk // pb)
                 if n_parts > 1:
-                    pml = scratch(n_items * n_parts * H * 32, torch.float32, q.device)
-                    po = scratch(n_items * n_parts * 16 * H * V, torch.float32, q.device)
+                    pml = scratch(n_items * n_parts * HQ * 32, torch.float32, q.device)
+                    po = scratch(n_items * n_parts * 16 * HQ * V, torch.float32, q.device)
             check(lib().k8s_masked_attn_mfma(ptr(q), ptr(kc), ptr(vt), ptr(seg.block_tables),
                                              seg.block_tables.shape[1], ptr(items), n_items, ptr(sink),
                                              ptr(gate), gs, ptr(out), H, G, D, V, BS, int(chunk), int(window),
                                              int(keep_first), float(scale), float(softcap), stream_ptr(q), pb, n_parts,
-                                             ptr(pml), ptr(po)), "masked_attn_mfma")
+                                             ptr(pml), ptr(po), int(maps), int(out_f32)), "masked_attn_mfma")
             return out
         check(lib().k8s_masked_attn_rows(ptr(q), ptr(kc), ptr(vc), ptr(seg.block_tables), seg.block_tables.shape[1],
                                          ptr(seg.row_seg), ptr(seg.seg_row0), ptr(seg.seg_pos0), ptr(sink), ptr(gate),
                                          gs, ptr(out), T, H, G, D, V, BS, int(chunk), int(window), int(keep_first),
-                                         float(scale), float(softcap), _dt(q.dtype), stream_ptr(q)),
-              "masked_attn_rows")
+                                         float(scale), float(softcap), _dt(q.dtype), stream_ptr(q), int(maps),
+                                         int(out_f32)), "masked_attn_rows")
         return out
-    kf, vf = kc.view(-1, G, D), vc.view(-1, G, V)
+    kf, vf = kc.view(-1, G, maps, D), vc.view(-1, G, V)
     rep = H // G
     for s in range(seg.n_seg):
         a, e, p0 = seg.row0_host[s], seg.row0_host[s + 1], seg.pos0_host[s]
         n, n_ctx = e - a, p0 + e - a
         kp = torch.arange(n_ctx)
         rows = seg.block_tables[s].long()[kp // BS] * BS + kp % BS
-        k = kf[rows].float().repeat_interleave(rep, 1)             # [ctx, H, D]
-        v = vf[rows].float().repeat_interleave(rep, 1)             # [ctx, H, V]
+        k = kf[rows].float().repeat_interleave(rep, 1).reshape(n_ctx, HQ, D)                  # [ctx, H M, D]
+        v = vf[rows].float().repeat_interleave(rep, 1).repeat_interleave(maps, 1)             # [ctx, H M, V]
         qi = (p0 + torch.arange(n))[:, None]
         vis = kp[None, :] <= qi
         if chunk > 0:
             vis &= (qi // chunk) == (kp[None, :] // chunk)
         if window > 0:
             vis &= ((qi - kp[None, :]) < window) | (kp[None, :] < keep_first)
-        sc = torch.einsum("thd,jhd->thj", q[a:e].float().view(n, H, D), k) * scale
+        sc = torch.einsum("thd,jhd->thj", q[a:e].float().view(n, HQ, D), k) * scale
         if softcap > 0:
             sc = softcap * torch.tanh(sc / softcap)
         sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
@@ -741,8 +818,8 @@ def masked_attention(q: torch.Tensor, H: int, G: int, D: int, V: int, kc: torch.
             den = den + torch.exp(sink[None, :, None] - m)
         o = torch.einsum("thj,jhv->thv", ex / den, v)
         if gate is not None:
-            o = o * torch.sigmoid(gate[a:e, :H])[:, :, None]
-        out[a:e] = o.reshape(n, H * V).to(q.dtype)
+            o = o * torch.sigmoid(gate[a:e, :HQ])[:, :, None]
+        out[a:e] = o.reshape(n, HQ * V).to(out.dtype)
     return out
 
 
@@ -758,26 +835,39 @@ def masked_mfma_ok(H: int, G: int, D: int, V: int, dtype, device) -> bool:
     return bool(fn(int(H), int(G), int(D), int(V))) if fn is not None else False
 
 
-def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, H: int, V: int, eps: float,
-                   out_dtype, mul: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``u / rms(u over each head's V) * w * sigmoid(gate)`` of fp32 rows ``o`` [T, H V], ``u = o * mul`` with ``mul``
-    [T, H] where given; ``w`` [V] (shared by the heads) or [H V]; ``gate`` [T, H V] fp32 (row stride free)."""
+def head_norm_gate(o: torch.Tensor, gate: Optional[torch.Tensor], w: Optional[torch.Tensor], H: int, V: int, eps: float,
+                   out_dtype, mul: Optional[torch.Tensor] = None, sub_lambda: Optional[float] = None,
+                   out_scale: float = 1.0) -> torch.Tensor:
+    """``u / rms(u over each head's V) * w * sigmoid(gate) * out_scale`` of fp32 rows ``o`` [T, H V], ``u = o * mul`` with
+    ``mul`` [T, H] where given; ``w`` [V] (shared by the heads) or [H V] or None; ``gate`` [T, H V] fp32 (row stride
+    free) or None.  With ``sub_lambda`` the rows hold two results per head, [T, H, 2, V], and
+    ``u = o[:, :, 0] - sub_lambda * o[:, :, 1]`` (two score maps over the same values, joined)."""
     T = o.shape[0]
     out = torch.empty(T, H * V, dtype=out_dtype, device=o.device)
+    sub = sub_lambda is not None
     if use_hip(o):
-        assert o.dtype == gate.dtype == w.dtype == torch.float32 and o.is_contiguous() and gate.stride(1) == 1
-        assert w.numel() in (V, H * V)
+        assert o.dtype == torch.float32 and o.is_contiguous() and o.shape[1] == H * V * (2 if sub else 1)
+        assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.shape[1] >= H * V)
+        assert w is None or (w.dtype == torch.float32 and w.numel() in (V, H * V))
         assert mul is None or (mul.dtype == torch.float32 and mul.is_contiguous() and mul.numel() == T * H)
-        check(lib().k8s_head_norm_gate(ptr(o), ptr(gate), gate.stride(0), ptr(w), V if w.numel() == H * V else 0,
-                                       ptr(out), T, H, V, float(eps), _dt(out_dtype), stream_ptr(o), ptr(mul)),
-              "head_norm_gate")
+        check(lib().k8s_head_norm_gate(ptr(o), ptr(gate), gate.stride(0) if gate is not None else 0, ptr(w),
+                                       V if w is not None and w.numel() == H * V else 0,
+                                       ptr(out), T, H, V, float(eps), _dt(out_dtype), stream_ptr(o), ptr(mul),
+                                       int(sub), float(sub_lambda or 0.0), float(out_scale)), "head_norm_gate")
         return out
-    oh = o.view(T, H, V)
+    if sub:
+        oh = o.view(T, H, 2, V)
+        oh = oh[:, :, 0] - sub_lambda * oh[:, :, 1]
+    else:
+        oh = o.view(T, H, V)
     if mul is not None:
         oh = oh * mul.view(T, H, 1)
-    oh = oh * torch.rsqrt(oh.pow(2).mean(-1, keepdim=True) + eps)
-    wv = w.view(H, V) if w.numel() == H * V else w.view(1, V)
-    out.copy_((oh * wv * torch.sigmoid(gate[:, :H * V]).view(T, H, V)).reshape(T, H * V).to(out_dtype))
+    oh = oh * torch.rsqrt(oh.pow(2).mean(-1, keepdim=True) + eps) * out_scale
+    if w is not None:
+        oh = oh * (w.view(H, V) if w.numel() == H * V else w.view(1, V))
+    if gate is not None:
+        oh = oh * torch.sigmoid(gate[:, :H * V]).view(T, H, V)
+    out.copy_(oh.reshape(T, H * V).to(out_dtype))
     return out
 
 
