@@ -12,6 +12,7 @@ import logging
 import math
 import os
 import threading
+import gc
 import time
 from typing import Callable, Dict, List, Optional, Sequence as Seq, Tuple
 
@@ -113,8 +114,17 @@ class GraphRunnerMixin:
             self._graph_pool = torch.cuda.graph_pool_handle()
         # thread_local: the graph-query batcher keeps issuing on its own stream from its
         # own thread while a bucket is captured mid-run
-        with torch.cuda.graph(graph, pool=self._graph_pool, capture_error_mode="thread_local"):
-            out = self._model_fwd(inp)
+        # no cyclic collection while the stream captures: a collector run that happens to start inside the
+        # capture would destroy graphs and free device memory of engines that are already gone, which a
+        # capturing stream does not allow (torch.cuda.graph collects once, before the capture begins)
+        gc_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, pool=self._graph_pool, capture_error_mode="thread_local"):
+                out = self._model_fwd(inp)
+        finally:
+            if gc_was_on:
+                gc.enable()
         self._graphs[key] = (graph, out)
         self.stats["captures"] += 1
         self.stats["capture_s"] += time.perf_counter() - t0
