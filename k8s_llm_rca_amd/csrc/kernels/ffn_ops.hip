@@ -75,6 +75,35 @@ __global__ void __launch_bounds__(256) glu_clamp_kernel(const TA* __restrict__ g
   stx(out, i, g / (1.f + expf(-alpha * g)) * (u + up_shift));
 }
 
+__device__ __forceinline__ void st8(uint16_t* p, size_t i, const float (&v)[8]) {
+  u16x8 raw;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) raw[k] = f2bf(v[k]);
+  *reinterpret_cast<u16x8*>(p + i) = raw;
+}
+__device__ __forceinline__ void st8(float* p, size_t i, const float (&v)[8]) {
+  *reinterpret_cast<f32x4*>(p + i) = f32x4{v[0], v[1], v[2], v[3]};
+  *reinterpret_cast<f32x4*>(p + i + 4) = f32x4{v[4], v[5], v[6], v[7]};
+}
+
+// The same for F a multiple of 8: eight neighbouring outputs per thread, 16-byte accesses.
+template <typename TA>
+__global__ void __launch_bounds__(256) glu_clamp8_kernel(const TA* __restrict__ gu, TA* __restrict__ out, size_t n8,
+                                                         int F, float alpha, float limit, float up_shift) {
+  const size_t i8 = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i8 >= n8) return;
+  const size_t i = i8 * 8, r = i / F, c = i - r * F;
+  float gv[8], uv[8], o[8];
+  ld8(gu, r * 2 * F + c, gv);
+  ld8(gu, r * 2 * F + F + c, uv);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const float g = fminf(gv[k], limit), u = fminf(fmaxf(uv[k], -limit), limit);
+    o[k] = g / (1.f + expf(-alpha * g)) * (u + up_shift);
+  }
+  st8(out, i, o);
+}
+
 // Router: one wave per token.  logits = Wr h in fp32; scores = sigmoid(logits)
 // (mode 0) or softmax (mode 1); the K largest (ties: lowest index), optionally
 // renormalised to sum 1 (divided by their sum + renorm_eps).  With `bias` [E] the
@@ -271,6 +300,12 @@ K8S_API int k8s_glu_clamp(const void* gu, void* out, int rows, int F, float alph
                           int dt, hipStream_t s) {
   const size_t n = (size_t)rows * F;
   if (n == 0) return 0;
+  if (F % 8 == 0 && ((uintptr_t)gu & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+    const size_t n8 = n / 8;
+    K8S_DT(dt, hipLaunchKernelGGL((glu_clamp8_kernel<TA>), dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, s,
+                                   (const TA*)gu, (TA*)out, n8, F, alpha, limit, up_shift));
+    return (int)hipGetLastError();
+  }
   K8S_DT(dt, hipLaunchKernelGGL((glu_clamp_kernel<TA>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
                                  (const TA*)gu, (TA*)out, n, F, alpha, limit, up_shift));
   return (int)hipGetLastError();

@@ -306,7 +306,9 @@ __device__ __forceinline__ bf16x8 mld16(const uint16_t* p) { return *reinterpret
 // SPLIT: workgroup z walks the blocks [z part_blocks, (z + 1) part_blocks) of its tile and leaves its maximum,
 // denominator and unnormalised output; masked_attn_merge_kernel joins the parts (and adds the sink).  Part
 // borders count blocks of the tile's own block list, so they depend on positions only.
-template <int NDC, int NV, int HW, bool CAP, bool SPLIT>
+// KH = 2 (two score maps per head, HW = 2): the wave's two query heads are the two maps of ONE head; each has its
+// own key head (its own key fragments) and both apply their weights to the same value fragments.
+template <int NDC, int NV, int HW, bool CAP, bool SPLIT, int KH = 1>
 __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   constexpr int D = NDC * 32, V = NV * 16;
   constexpr float kLog2e = 1.4426950408889634f;
@@ -371,9 +373,9 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   // loads and value loads are dependent memory accesses, so they are issued a block ahead into the SAME
   // registers: the next keys as soon as this block's scores are formed, the next values as soon as this
   // block's value products are issued; the softmax and the products run meanwhile.
-  // (with score maps, HW = 1: map m of a head reads key head m of its group and the group's one value head)
+  // (with score maps: map m of a head reads key head m of its group and the group's one value head)
   const int gv = h0 / a.M / hpg, g = gv * a.M + h0 % a.M;
-  bf16x8 kf[2][NDC];
+  bf16x8 kf[KH][2][NDC];
   bf16x8 vf[NV];
   auto block_at = [&](int bi) { return bi < nblkA ? a_beg + 32 * bi : lo_al + 32 * (bi - nblkA); };
   // lane i of (kbv, pgv, ofv) holds the first key, the page and the offset within the page of block
@@ -392,11 +394,13 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
   auto load_k = [&](int page, int off) {
     const uint16_t* kp = a.kc + ((size_t)page * a.BS + off) * NK + g * D + 8 * hq;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int key = 8 * (r >> 2) + 4 * t + (r & 3);
+    for (int kh = 0; kh < KH; ++kh)
 #pragma unroll
-      for (int cc = 0; cc < NDC; ++cc) kf[t][cc] = mld16(kp + (size_t)key * NK + 32 * cc);
-    }
+      for (int t = 0; t < 2; ++t) {
+        const int key = 8 * (r >> 2) + 4 * t + (r & 3);
+#pragma unroll
+        for (int cc = 0; cc < NDC; ++cc) kf[kh][t][cc] = mld16(kp + (size_t)key * NK + kh * D + 32 * cc);
+      }
   };
   auto load_v = [&](int page, int off) {
     const uint16_t* vp = a.vt + ((size_t)page * NVt + (size_t)gv * V) * a.BS + off + 8 * hq;
@@ -423,7 +427,7 @@ __global__ void __launch_bounds__(512) masked_attn_mfma_kernel(MaskArgs a) {
         f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int cc = 0; cc < NDC; ++cc)
-          sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][cc], qf[hh][cc], sacc, 0, 0, 0);
+          sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[KH == 1 ? 0 : hh][t][cc], qf[hh][cc], sacc, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) p[hh][4 * t + i] = sacc[i];
       }
@@ -561,29 +565,32 @@ __global__ void __launch_bounds__(256) masked_attn_merge_kernel(MaskArgs a, int 
   }
 }
 
-template <int NDC, int NV, int HW, bool CAP>
+template <int NDC, int NV, int HW, bool CAP, int KH>
 static int launch_mask_cap(const MaskArgs& a, int n_items, hipStream_t s) {
   const int waves_all = (a.H + HW - 1) / HW;               // HW heads per wave, up to eight waves per workgroup
   const int gy = (waves_all + 7) / 8, waves = gy > 1 ? 8 : waves_all;
   if (a.n_parts > 1) {
-    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, CAP, true>), dim3(n_items, gy, a.n_parts), dim3(64 * waves),
-                       0, s, a);
+    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, CAP, true, KH>), dim3(n_items, gy, a.n_parts),
+                       dim3(64 * waves), 0, s, a);
     hipLaunchKernelGGL(masked_attn_merge_kernel, dim3(n_items, 8), dim3(256), 0, s, a, NV * 16);
   } else {
-    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, CAP, false>), dim3(n_items, gy), dim3(64 * waves), 0, s, a);
+    hipLaunchKernelGGL((masked_attn_mfma_kernel<NDC, NV, HW, CAP, false, KH>), dim3(n_items, gy), dim3(64 * waves), 0, s,
+                       a);
   }
   return (int)hipGetLastError();
 }
 
-template <int NDC, int NV, int HW>
+template <int NDC, int NV, int HW, int KH = 1>
 static int launch_mask_hw(const MaskArgs& a, int n_items, hipStream_t s) {
-  return a.softcap > 0.f ? launch_mask_cap<NDC, NV, HW, true>(a, n_items, s)
-                         : launch_mask_cap<NDC, NV, HW, false>(a, n_items, s);
+  if (KH == 1 && a.softcap > 0.f) return launch_mask_cap<NDC, NV, HW, true, 1>(a, n_items, s);
+  return launch_mask_cap<NDC, NV, HW, false, KH>(a, n_items, s);
 }
 
-// two heads per wave where the heads of a key / value head come in pairs, else one
+// two heads per wave where the heads of a key / value head come in pairs, or where a head has two score maps
+// (uncapped: the pair is the head's two maps, which share their values); else one
 template <int NDC, int NV>
 static int launch_mask_mfma(const MaskArgs& a, int n_items, hipStream_t s) {
+  if (a.M == 2 && !(a.softcap > 0.f)) return launch_mask_hw<NDC, NV, 2, 2>(a, n_items, s);
   return a.M == 1 && (a.H / a.G) % 2 == 0 ? launch_mask_hw<NDC, NV, 2>(a, n_items, s)
                                           : launch_mask_hw<NDC, NV, 1>(a, n_items, s);
 }

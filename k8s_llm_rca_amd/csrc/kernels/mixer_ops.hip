@@ -273,7 +273,8 @@ __global__ void __launch_bounds__(128) scan_carry_kernel(const float* __restrict
 // x (row stride xs), bc rows (stride bs: B [G][N] | C [G][N]) and z (stride zs) have type TA; dtp (stride dts) is
 // fp32; y [T][C] fp32.  state [slots][C][N].  EX picks the exponentials (DecayExp).  MODE 0 / 1 / 2 and the chunk
 // arrays as in selective_scan_kernel; a chunk's decay is exp(-rate * sum dt), kept per (chunk, channel) in csd.
-template <int NMAX, int MODE, typename TA, typename EX>
+// VEC (fp32 inputs, N a multiple of 4, rows 16-byte aligned): B and C are read four states per load.
+template <int NMAX, int MODE, typename TA, typename EX, bool VEC = false>
 __global__ void __launch_bounds__(128) ssd_scan_kernel(const TA* __restrict__ x, int xs, const TA* __restrict__ bc, int bs,
                                                        const float* __restrict__ dtp, int dts,
                                                        const float* __restrict__ dt_bias, const float* __restrict__ rate,
@@ -314,12 +315,29 @@ __global__ void __launch_bounds__(128) ssd_scan_kernel(const TA* __restrict__ x,
     const TA* Cp = Bp + (size_t)G * N;
     float acc = 0.f;
     sd += dt;
+    if (VEC) {
+      const f32x4* B4 = reinterpret_cast<const f32x4*>(Bp);
+      const f32x4* C4 = reinterpret_cast<const f32x4*>(Cp);
 #pragma unroll
-    for (int n = 0; n < NMAX; ++n)
-      if (n < N) {
-        S[n] = fmaf(a, S[n], dx * ldm(Bp, n));
-        if (MODE != 1) acc = fmaf(S[n], ldm(Cp, n), acc);
-      }
+      for (int n4 = 0; n4 < NMAX / 4; ++n4)
+        if (4 * n4 < N) {
+          const f32x4 b = B4[n4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) S[4 * n4 + k] = fmaf(a, S[4 * n4 + k], dx * b[k]);
+          if (MODE != 1) {
+            const f32x4 cv = C4[n4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) acc = fmaf(S[4 * n4 + k], cv[k], acc);
+          }
+        }
+    } else {
+#pragma unroll
+      for (int n = 0; n < NMAX; ++n)
+        if (n < N) {
+          S[n] = fmaf(a, S[n], dx * ldm(Bp, n));
+          if (MODE != 1) acc = fmaf(S[n], ldm(Cp, n), acc);
+        }
+    }
     if (MODE != 1) y[(size_t)r * C + c] = (acc + Dc * xv) * EX::silu(ldm(z, (size_t)r * zs + c));
   }
   if (MODE != 2) {
@@ -623,10 +641,17 @@ K8S_API int k8s_ssd_scan(const void* x, int xs, const void* bc, int bs, int dt, 
   if (T <= 0 || n_seg <= 0) return 0;
   if (N < 1 || N > 128 || H < 1 || P < 1 || G < 1 || H % G) return (int)hipErrorInvalidValue;
   const int C = H * P, cb = (C + 127) / 128, hpg = H / G;
+  const bool vec = dt == 1 && N % 4 == 0 && bs % 4 == 0 && ((uintptr_t)bc & 15) == 0;
 #define K8S_SSD_E(NM, MODE, items, EX)                                                                            \
-  K8S_MDT(dt, hipLaunchKernelGGL((ssd_scan_kernel<NM, MODE, TA, EX>), dim3(items, cb), dim3(128), 0, s,           \
-                                 (const TA*)x, xs, (const TA*)bc, bs, dtp, dts, dt_bias, rate, D, (const TA*)z,   \
-                                 zs, state, seg_row0, seg_pos0, seg_slot, y, C, N, P, hpg, G, chunks, cs, csd))
+  if (vec) {                                                                                                      \
+    hipLaunchKernelGGL((ssd_scan_kernel<NM, MODE, float, EX, true>), dim3(items, cb), dim3(128), 0, s,            \
+                       (const float*)x, xs, (const float*)bc, bs, dtp, dts, dt_bias, rate, D, (const float*)z, zs, \
+                       state, seg_row0, seg_pos0, seg_slot, y, C, N, P, hpg, G, chunks, cs, csd);                 \
+  } else {                                                                                                        \
+    K8S_MDT(dt, hipLaunchKernelGGL((ssd_scan_kernel<NM, MODE, TA, EX>), dim3(items, cb), dim3(128), 0, s,         \
+                                   (const TA*)x, xs, (const TA*)bc, bs, dtp, dts, dt_bias, rate, D, (const TA*)z, \
+                                   zs, state, seg_row0, seg_pos0, seg_slot, y, C, N, P, hpg, G, chunks, cs, csd)) \
+  }
 #define K8S_SSD_M(NM, MODE, items)                \
   if (fast) {                                     \
     K8S_SSD_E(NM, MODE, items, DecayExp<uint16_t>) \

@@ -210,26 +210,26 @@ class PumozenConfig:
 
 def _stack(n_groups: int, W: int, heads: int, kv_heads: int, dim: int, ff: int, experts: int, state: int):
     """Groups of (mamba2 + dense, attention_2 + experts, attention + dense, attention_2 on the first one's pages +
-    experts)."""
+    experts).  The two-map attention has half the head size for its scores and the full one for its values."""
     dense = FfSpec("dense", ff, 7.0)
-    moe = FfSpec("moe", ff // 4, 7.0, experts, 2, 1.5, ff // 2, 7.0)
+    moe = FfSpec("moe", ff // 4, 7.0, experts, 2, 1.5, ff // 4, 7.0)
     out = []
     for g in range(n_groups):
         b = 4 * g
+        two = dict(heads=heads, kv_heads=kv_heads, dim=dim // 2, vdim=dim, scale=1.0 / math.sqrt(dim // 2), diff=0.6,
+                   temp_coef=0.2, temp_every=512)
         out += [LayerSpec("mamba2", ssd=SsdSpec(2 * W // 64, 64, state, max(1, heads // 8), 4, 2), mlp=dense),
-                LayerSpec("attention_2", diff=DiffAttnSpec(heads // 2, max(1, kv_heads // 2), dim, 2 * dim,
-                                                           1.0 / math.sqrt(dim), 0.6, 0.2, 512), mlp=moe),
+                LayerSpec("attention_2", diff=DiffAttnSpec(**two), mlp=moe),
                 LayerSpec("attention", attn=SinkAttnSpec(heads, kv_heads, dim, dim, 1.0 / math.sqrt(dim), dim // 2,
                                                          500000.0), mlp=dense),
-                LayerSpec("attention_2", diff=DiffAttnSpec(heads // 2, max(1, kv_heads // 2), dim, 2 * dim,
-                                                           1.0 / math.sqrt(dim), 0.6, 0.2, 512, kv_from=b + 1), mlp=moe)]
+                LayerSpec("attention_2", diff=DiffAttnSpec(kv_from=b + 1, **two), mlp=moe)]
     return tuple(out)
 
 
 PRESETS: Dict[str, PumozenConfig] = {
     "tiny-pumozen": PumozenConfig("tiny-pumozen", 8192, 256, _stack(1, 256, 4, 2, 32, 512, 4, 16), side_dim=16),
     # sizes of a ~1B-class decoder's layers (benchmarks; random weights)
-    "pumozen-1b": PumozenConfig("pumozen-1b", 32768, 2048, _stack(3, 2048, 16, 4, 128, 8192, 8, 64), side_dim=256),
+    "pumozen-1b": PumozenConfig("pumozen-1b", 32768, 2048, _stack(3, 2048, 16, 2, 128, 8192, 8, 64), side_dim=256),
 }
 
 

@@ -521,9 +521,10 @@ def test_state_space_scan_across_portions_and_slots(backend, H, P, G, Ns, T):
     column slices of wider matrices, as the layer hands them over."""
     dev, dt = backend
     C = H * P
-    wide = rnd(T, C + 2 * G * Ns + 3, seed=P).to(torch.bfloat16).double()
+    ld = 4 if Ns % 4 == 0 and C % 4 == 0 else 1       # 4: B and C rows are 16-byte aligned (the four-wide loads)
+    wide = rnd(T, ld + C + 2 * G * Ns + (4 if ld == 4 else 2), seed=P).to(torch.bfloat16).double()
     zd = rnd(T, C + H + 2, seed=2).to(torch.bfloat16).double()
-    x, bc, z, dtp = wide[:, 1:1 + C], wide[:, 1 + C:1 + C + 2 * G * Ns], zd[:, :C], zd[:, C + 1:C + 1 + H]
+    x, bc, z, dtp = wide[:, ld:ld + C], wide[:, ld + C:ld + C + 2 * G * Ns], zd[:, :C], zd[:, C + 1:C + 1 + H]
     dt_bias, rate, Dk = rnd(H, seed=3) - 0.5, torch.exp(rnd(H, seed=4, std=0.5)), rnd(H, seed=5) + 1.0
     want, Sw = ssd_reference(x, bc, dtp, dt_bias, rate, Dk, z, H, P, G, Ns)
     wd, zf = wide.to(dev).to(dt), zd.to(dev).to(dt)
@@ -532,7 +533,7 @@ def test_state_space_scan_across_portions_and_slots(backend, H, P, G, Ns, T):
         state = torch.full((3, C, Ns), float("nan"), device=dev)
 
         def run(s, e):
-            return S.ssd_scan(wd[s:e, 1:1 + C], wd[s:e, 1 + C:1 + C + 2 * G * Ns], dtf[s:e, C + 1:C + 1 + H],
+            return S.ssd_scan(wd[s:e, ld:ld + C], wd[s:e, ld + C:ld + C + 2 * G * Ns], dtf[s:e, C + 1:C + 1 + H],
                               f32(dt_bias, dev), f32(rate, dev), f32(Dk, dev), zf[s:e, :C], H, P, G, Ns, state,
                               seg_meta([e - s], [s], [1], dev), fast_exp=dt == torch.bfloat16)
         got = in_portions(run, T, cuts)
