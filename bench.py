@@ -6,7 +6,7 @@ Contract: ``python bench.py --gpus N --steps K --warmup W``.  Under torchrun
 the N rank processes itself (one per GPU, data-parallel engine replicas).
 Rank 0 prints ONE JSON line.  See k8s_llm_rca_amd/bench/rca_bench.py.
 
-``python bench.py --model-throughput zasapel-1b,ligipel-1b,mixtral-1b,lizesun-1b,llama-1b [--shapes 8x2048]``
+``python bench.py --model-throughput zasapel-1b,ligipel-1b,mixtral-1b,lizesun-1b,llama-1b,pumozen-1b [--shapes 8x2048]``
 measures prefill and decode tokens/s of model presets side by side instead
 (k8s_llm_rca_amd/bench/model_bench.py); without that flag nothing changes.
 """

@@ -1,5 +1,6 @@
 """Prefill and decode throughput of one or more model presets, side by side
-(``python bench.py --model-throughput zasapel-1b,ligipel-1b,mixtral-1b``, ``... lizesun-1b,llama-1b``).
+(``python bench.py --model-throughput zasapel-1b,ligipel-1b,mixtral-1b``, ``... lizesun-1b,llama-1b``,
+``... pumozen-1b,ligipel-1b``).
 
 Random weights, one GPU, the engine's own step (``LLMEngine.feed``: given
 tokens, no sampling): a prefill step is ``batch`` prompts of ``seq`` tokens in

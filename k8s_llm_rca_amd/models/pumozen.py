@@ -46,6 +46,7 @@ from ..ops import norm as N
 from ..ops import seq_ops as S
 from ..ops.linear import linear, linear_f32out
 from ..parallel.groups import ParallelContext, single
+from .moe import MoELayerSet
 
 GLU_ALPHA = 1.702       # g * sigmoid(GLU_ALPHA g) * (u + 1)
 RENORM_EPS = 1e-20      # chosen scores / (their sum + RENORM_EPS)
@@ -481,8 +482,19 @@ class PumozenModel:
         w, ids = r[0], r[1]
         order, inv, offsets = M.align(ids, f.experts)
         xp = M.gather_rows(h, order, f.top)
-        act = self._unit(M.grouped_auto(xp, L["w13"], offsets), f.limit)
-        yp = M.grouped_auto(act, L["w2"], offsets)
+        rows = xp.shape[0]
+        dev16 = xp.is_cuda and xp.dtype == torch.bfloat16
+        if dev16 and rows <= MoELayerSet.GLDS_MAX_ROWS:
+            # decode sizes: the weight-streaming kernels the Mixtral block runs there (LDS-DMA strips for
+            # gate | up; the down projection below with its K split over workgroups)
+            gu = M.grouped_gemm(xp, L["w13"], offsets, glds=MoELayerSet.GLDS_UP[0], splits=MoELayerSet.GLDS_UP[1])
+        else:
+            gu = M.grouped_auto(xp, L["w13"], offsets)
+        act = self._unit(gu, f.limit)
+        if dev16 and rows <= MoELayerSet.SPLIT_MAX_ROWS:
+            yp = M.grouped_gemm(act, L["w2"], offsets, splits=MoELayerSet.DOWN_SPLITS)
+        else:
+            yp = M.grouped_auto(act, L["w2"], offsets)
         routed = M.combine_f32(yp, inv, T, f.top, w)
         if not f.shared_ff:
             return routed, None, None

@@ -731,6 +731,8 @@ OTHER = {
                           (dif(heads=4, kv_heads=2, dim=64, vdim=64, kv_from=0), None),
                           (dif(heads=3, kv_heads=1, dim=128, vdim=128, every=0), dense()),
                           (att(heads=4, kv_heads=2, dim=128, rot=64, kv_from=1), None), (att(heads=3, kv_heads=3, dim=64, rot=0), None)],
+    "expert_kernel_sizes": [(dif(), moe(ff=128, experts=4, top=2, shared=128)), (mam(), moe(ff=64, experts=3, top=1, shared=0)),
+                            (att(), dense(ff=256))],
     "one_head_everywhere": [(att(heads=1, kv_heads=1, dim=4, rot=2), dense(ff=8)), (dif(heads=1, kv_heads=1), moe(experts=1, top=1)),
                             (mam(heads=1, vdim=4, groups=1, norm_groups=1), None)],
     "top_one_and_top_all": [(mam(), moe(experts=4, top=1, scale=1.0)), (att(), moe(experts=4, top=4, scale=0.5, shared=0))],
@@ -750,7 +752,7 @@ OTHER = {
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("name", sorted(OTHER))
 def test_other_sizes(backend, name):
-    d = config(OTHER[name], width={"unaligned_sizes": 34, "matrix_core_sizes": 64}.get(name, 40), eps=1e-3,
+    d = config(OTHER[name], width={"unaligned_sizes": 34, "matrix_core_sizes": 64, "expert_kernel_sizes": 128}.get(name, 40), eps=1e-3,
                side={"no_shared_no_side_no_mlp": 0, "unaligned_sizes": 5, "one_head_everywhere": 1}.get(name, 8))
     W = weights(d, 11)
     tokens = toks(40, d["vocab"], 12)
