@@ -1,14 +1,15 @@
-"""Pumozen decoder: sublayers that read the fp32 residual ITSELF and are normed on their way back,
+"""Pumozen decoder: post-sublayer norms -- each sublayer reads the raw fp32 residual and only its result is normed,
 
     x <- x + LN1(mixer(x));   x <- x + LN2(ff(x));   x <- x + rms(side_i(x, token)) w_side
 
 with layer norms (weight and bias) on the sublayer outputs, three kinds of mixer, a dense or mixture-of-experts
 feed-forward, and a per-layer token input behind the feed-forward.
 
-``attention``:    q = W_q x, k = W_k x, and the VALUES ARE THE KEYS as projected (no W_v).  q and k are RMS-normed
-                  over their whole projection (all heads at once, a weight of that size), then rotated on the first
-                  ``rot.dims`` entries of every head (rotate-half pairs); causal softmax with a sink of score 0 in
-                  the denominator.
+``attention``:    q = W_q x, k = W_k x; keys double as values: what is cached as the value is the key projection
+                  itself, taken in front of its norm and rotation (there is no value projection).  q and k get one
+                  RMS norm each across ALL their heads (a weight as wide as the projection), then the rotation on
+                  the first ``rot.dims`` entries of every head (rotate-half pairs); causal softmax whose denominator
+                  holds one extra term e^0 (a sink without a value).
 ``mamba2``:       state-space duality: one projection gives ``z | x | B | C | dt``; ``x | B | C`` pass a short causal
                   convolution with bias and SiLU; ``dt = softplus(dt + dt_bias)``; per head
                   ``S <- exp(-e^(A_log) dt) S + dt B x^T``, ``y = S^T C + D x``; ``y silu(z)`` is RMS-normed in
@@ -54,7 +55,7 @@ RENORM_EPS = 1e-20      # chosen scores / (their sum + RENORM_EPS)
 
 @dataclass(frozen=True)
 class SinkAttnSpec:
-    """``attention``: values are the keys as projected (``vdim == dim``)."""
+    """``attention``: keys double as values (``vdim == dim``)."""
     heads: int
     kv_heads: int
     dim: int

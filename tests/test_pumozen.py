@@ -321,14 +321,14 @@ def test_preparation_with_a_norm_over_the_whole_projection(backend, H, G, D, rot
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("H,G,D,V,every", [(4, 2, 8, 12, 7), (3, 3, 6, 5, 1), (2, 1, 16, 8, 0), (1, 1, 70, 3, 256),
+@pytest.mark.parametrize("H,G,D,V,every", [(4, 2, 8, 12, 7), (3, 3, 6, 5, 1), (2, 1, 16, 8, 0), (1, 1, 70, 3, 200),
                                            (2, 0, 8, 4, 3)])
 def test_preparation_of_two_score_maps(backend, H, G, D, V, every):
     """Every (head, map) of q and k normed by itself with one shared weight; the query temperature steps with
     floor((p + 1) / every); values behind the keys."""
     dev, dt = backend
     T, BS, eps, coef = 9, 8, 1e-3, 0.45
-    pos = torch.tensor([0, 1, 5, 6, 7, 13, 254, 255, 70003])
+    pos = torch.tensor([0, 1, 5, 6, 7, 13, 198, 199, 70003])
     nq, nk, nv = 2 * H * D, 2 * G * D, G * V
     x = rnd(T, nq + nk + nv + 2, seed=H + D, std=2.0)
     qw, kw = rnd(D, seed=4) + 1.5, rnd(D, seed=5) + 1.5
